@@ -1,0 +1,252 @@
+"""ctypes bindings of the checker libraries (TEST INFRASTRUCTURE ONLY).
+
+`oracle()` loads oracle/libfkoracle.so, the plain-C restatement of the reference's CPU executor
+(fk_oracle.c); `reference()` loads oracle/_ref/libfkref.so, the reference's own headers compiled for
+its CPU backend (ref_driver.cpp), or returns None when that build is absent.  Both are built by
+oracle/Makefile.  Only tests, the smoke check and the CPU-baseline leg of the benchmark import this
+module; the shipped library never does.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+PRESERVE_AR, IGNORE_AR, PRESERVE_AR_RN_EVEN, PRESERVE_AR_LEFT = 0, 1, 2, 3
+
+
+class Rect(C.Structure):
+    _fields_ = [("x", C.c_int), ("y", C.c_int), ("width", C.c_int), ("height", C.c_int)]
+
+
+class ResizeParams(C.Structure):
+    _fields_ = [("dst_w", C.c_int), ("dst_h", C.c_int), ("fx", C.c_float), ("fy", C.c_float),
+                ("src_w", C.c_int), ("src_h", C.c_int), ("x1", C.c_int), ("y1", C.c_int),
+                ("x2", C.c_int), ("y2", C.c_int)]
+
+
+def rect_array(rects):
+    arr = (Rect * len(rects))()
+    for i, r in enumerate(rects):
+        arr[i] = Rect(*[int(v) for v in r])
+    return arr
+
+
+def _f3(v):
+    return (C.c_float * 3)(*[float(x) for x in v])
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+_u8p, _f32p, _sz, _i, _f = C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_float
+_f3p = C.POINTER(C.c_float)
+_rp = C.POINTER(Rect)
+
+_CHAIN_SIGS = {
+    # name: (argtypes for the oracle; the reference driver has the same minus the quirk flag)
+    "crop_resize_muls_bgr_tensor": [_u8p, _i, _i, _sz, _rp, _i, _i, _i, _i, _f3p, _f3p, _f3p, _f3p, _i, _f32p],
+    "muladd_chain_f32c3": [_f32p, _i, _i, _sz, _i, _f, _f, _f32p, _sz],
+    "single_op_f32c3": [_f32p, _i, _i, _sz, _i, _f, _f32p, _sz],
+    "batch_crop_resize_norm_split": [C.POINTER(C.c_void_p), _i, _i, _sz, _rp, _i, _i, _i, _f3p, _f3p, _f3p, _i, _f32p],
+    "resize_crop_tiles": [_u8p, _i, _i, _sz, _i, _i, _rp, _i, _i, _i, _f3p, _i, _f32p],
+    "rgba2gray_u8c4": [_u8p, _i, _i, _sz, _u8p, _sz],
+    "resize_mul_u8c4_f32c4": [_u8p, _i, _i, _sz, _i, _i, _f, _i, _f32p, _sz],
+    "crop_mul_saturate_u8c4": [_u8p, _i, _i, _sz, Rect, _i, _u8p, _sz],
+    "rgba2bgr_sub_u8c4_f32c3": [_u8p, _i, _i, _sz, _f, _f32p, _sz],
+    "batch_crop_cast_tensor": [_u8p, _i, _i, _sz, _rp, _i, _i, _i, _i, _f32p],
+}
+# position of the quirk / exec_all flag that the reference driver's signature does not have
+_ORACLE_ONLY_ARG = {
+    "crop_resize_muls_bgr_tensor": 13, "batch_crop_resize_norm_split": 11, "resize_crop_tiles": 11,
+    "resize_mul_u8c4_f32c4": 7, "batch_crop_cast_tensor": 8,
+}
+
+
+def build(with_reference=True):
+    """(Re)build the checker libraries with oracle/Makefile."""
+    target = "all" if with_reference else "libfkoracle.so"
+    subprocess.run(["make", "-C", _HERE, target], check=True, stdout=subprocess.DEVNULL)
+
+
+class _Lib:
+    """Thin numpy-facing wrapper; `ref=True` talks to the reference driver (literal host semantics)."""
+
+    def __init__(self, cdll, ref):
+        self.c = cdll
+        self.ref = ref
+        pre = "fkr_" if ref else "fko_"
+        for name, sig in _CHAIN_SIGS.items():
+            fn = getattr(cdll, pre + name)
+            sig = list(sig)
+            if ref and name in _ORACLE_ONLY_ARG:
+                del sig[_ORACLE_ONLY_ARG[name]]
+            fn.argtypes = sig
+            fn.restype = C.c_int if ref else None
+        if ref:
+            cdll.fkr_cxp_round.argtypes = [_f]
+            cdll.fkr_cxp_round.restype = _f
+            cdll.fkr_saturate_float_to_u8.argtypes = [_f]
+            cdll.fkr_saturate_float_to_u8.restype = C.c_uint8
+            cdll.fkr_saturate_int_to_u8.argtypes = [_i]
+            cdll.fkr_saturate_int_to_u8.restype = C.c_uint8
+            cdll.fkr_rgb2gray_u8.argtypes = [C.c_uint8] * 3
+            cdll.fkr_rgb2gray_u8.restype = C.c_uint8
+        else:
+            cdll.fko_fill_bytes.argtypes = [C.c_uint64, C.c_void_p, _sz]
+            cdll.fko_fill_unit_floats.argtypes = [C.c_uint64, C.c_void_p, _sz]
+            cdll.fko_fill_uniform_ints.argtypes = [C.c_uint64, _i, _i, C.c_void_p, _sz]
+            cdll.fko_fill_gradient_noise_u8c3.argtypes = [C.c_uint64, C.c_void_p, _i, _i]
+            cdll.fko_fnv1a64.argtypes = [C.c_void_p, _sz]
+            cdll.fko_fnv1a64.restype = C.c_uint64
+            cdll.fko_round.argtypes = [_f]
+            cdll.fko_round.restype = _f
+            cdll.fko_resize_build.argtypes = [_i, _i, _i, _i, _i, C.POINTER(ResizeParams)]
+            cdll.fko_bilinear_u8.argtypes = [_u8p, _sz, _i, _i, _i, _i, _i, _f, _f, _i, _f32p]
+            cdll.fko_saturate_int_to_u8.argtypes = [_i]
+            cdll.fko_saturate_int_to_u8.restype = C.c_uint8
+            cdll.fko_saturate_float_to_u8.argtypes = [_f]
+            cdll.fko_saturate_float_to_u8.restype = C.c_uint8
+            cdll.fko_rgb2gray_u8.argtypes = [C.c_uint8] * 3
+            cdll.fko_rgb2gray_u8.restype = C.c_uint8
+
+    def _call(self, name, args):
+        args = list(args)
+        if self.ref and name in _ORACLE_ONLY_ARG:
+            del args[_ORACLE_ONLY_ARG[name]]
+        rc = getattr(self.c, ("fkr_" if self.ref else "fko_") + name)(*args)
+        if self.ref and rc != 0:
+            raise ValueError("reference driver has no instantiation for this batch size / depth")
+
+    # ---- generators (oracle library only) ----
+    def bytes(self, seed, shape):
+        out = np.empty(shape, np.uint8)
+        self.c.fko_fill_bytes(seed, _p(out), out.size)
+        return out
+
+    def unit_floats(self, seed, shape):
+        out = np.empty(shape, np.float32)
+        self.c.fko_fill_unit_floats(seed, _p(out), out.size)
+        return out
+
+    def uniform_ints(self, seed, lo, hi, n):
+        out = np.empty(n, np.int32)
+        self.c.fko_fill_uniform_ints(seed, lo, hi, _p(out), n)
+        return out
+
+    def gradient_noise_u8c3(self, seed, w, h):
+        out = np.empty((h, w, 3), np.uint8)
+        self.c.fko_fill_gradient_noise_u8c3(seed, _p(out), w, h)
+        return out
+
+    def fnv1a64(self, a):
+        a = np.ascontiguousarray(a)
+        return int(self.c.fko_fnv1a64(_p(a), a.nbytes))
+
+    def resize_build(self, aspect, src_w, src_h, dst_w, dst_h):
+        p = ResizeParams()
+        self.c.fko_resize_build(aspect, src_w, src_h, dst_w, dst_h, C.byref(p))
+        return p
+
+    def bilinear_u8(self, img, org, src_size, sx, sy, quirk=0):
+        h, w, cn = img.shape
+        out = np.empty(cn, np.float32)
+        self.c.fko_bilinear_u8(_p(img), img.strides[0], cn, org[0], org[1], src_size[0], src_size[1],
+                               float(sx), float(sy), quirk, _p(out))
+        return out
+
+    # ---- chains: images are (h, w, c) arrays whose row stride is the pitch ----
+    def crop_resize_muls_bgr_tensor(self, src, rects, dst, aspect, background, mul, sub, div, quirk=0):
+        h, w, _ = src.shape
+        out = np.empty((len(rects), dst[1], dst[0], 3), np.float32)
+        self._call("crop_resize_muls_bgr_tensor",
+                   [_p(src), w, h, src.strides[0], rect_array(rects), len(rects), dst[0], dst[1], aspect,
+                    _f3(background), _f3(mul), _f3(sub), _f3(div), quirk, _p(out)])
+        return out
+
+    def muladd_chain_f32c3(self, src, depth, mul_v, add_v):
+        h, w, _ = src.shape
+        out = np.empty((h, w, 3), np.float32)
+        self._call("muladd_chain_f32c3", [_p(src), w, h, src.strides[0], depth, mul_v, add_v, _p(out), out.strides[0]])
+        return out
+
+    def single_op_f32c3(self, src, is_add, v):
+        h, w, _ = src.shape
+        out = np.empty((h, w, 3), np.float32)
+        self._call("single_op_f32c3", [_p(src), w, h, src.strides[0], int(is_add), v, _p(out), out.strides[0]])
+        return out
+
+    def batch_crop_resize_norm_split(self, srcs, rects, dst, div1, sub, div2, quirk=0):
+        n = len(srcs)
+        h, w, _ = srcs[0].shape
+        ptrs = (C.c_void_p * n)(*[s.ctypes.data for s in srcs])
+        out = np.empty((n, 3, dst[1], dst[0]), np.float32)
+        self._call("batch_crop_resize_norm_split",
+                   [ptrs, w, h, srcs[0].strides[0], rect_array(rects), n, dst[0], dst[1], _f3(div1), _f3(sub),
+                    _f3(div2), quirk, _p(out)])
+        return out
+
+    def resize_crop_tiles(self, src, resized, rects, tile, mul, quirk=0):
+        h, w, _ = src.shape
+        out = np.empty((len(rects), tile[1], tile[0], 3), np.float32)
+        self._call("resize_crop_tiles",
+                   [_p(src), w, h, src.strides[0], resized[0], resized[1], rect_array(rects), len(rects), tile[0],
+                    tile[1], _f3(mul), quirk, _p(out)])
+        return out
+
+    def rgba2gray_u8c4(self, src):
+        h, w, _ = src.shape
+        out = np.empty((h, w), np.uint8)
+        self._call("rgba2gray_u8c4", [_p(src), w, h, src.strides[0], _p(out), out.strides[0]])
+        return out
+
+    def resize_mul_u8c4_f32c4(self, src, dst, mul_v, quirk=0):
+        h, w, _ = src.shape
+        out = np.empty((dst[1], dst[0], 4), np.float32)
+        self._call("resize_mul_u8c4_f32c4", [_p(src), w, h, src.strides[0], dst[0], dst[1], mul_v, quirk, _p(out), out.strides[0]])
+        return out
+
+    def crop_mul_saturate_u8c4(self, src, rect, mul_v):
+        h, w, _ = src.shape
+        out = np.empty((rect[3], rect[2], 4), np.uint8)
+        self._call("crop_mul_saturate_u8c4", [_p(src), w, h, src.strides[0], Rect(*rect), mul_v, _p(out), out.strides[0]])
+        return out
+
+    def rgba2bgr_sub_u8c4_f32c3(self, src, sub_v):
+        h, w, _ = src.shape
+        out = np.empty((h, w, 3), np.float32)
+        self._call("rgba2bgr_sub_u8c4_f32c3", [_p(src), w, h, src.strides[0], sub_v, _p(out), out.strides[0]])
+        return out
+
+    def batch_crop_cast_tensor(self, src, rects, max_size, exec_all=1, fill=None):
+        h, w, _ = src.shape
+        out = np.empty((len(rects), max_size[1], max_size[0], 3), np.float32)
+        if fill is not None:
+            out[...] = fill
+        self._call("batch_crop_cast_tensor",
+                   [_p(src), w, h, src.strides[0], rect_array(rects), len(rects), max_size[0], max_size[1],
+                    exec_all, _p(out)])
+        return out
+
+
+_cache = {}
+
+
+def oracle():
+    if "o" not in _cache:
+        path = os.path.join(_HERE, "libfkoracle.so")
+        if not os.path.exists(path):
+            build(with_reference=False)
+        _cache["o"] = _Lib(C.CDLL(path), ref=False)
+    return _cache["o"]
+
+
+def reference():
+    """The reference-headers build, or None when oracle/_ref/libfkref.so has not been built."""
+    if "r" not in _cache:
+        path = os.path.join(_HERE, "_ref", "libfkref.so")
+        _cache["r"] = _Lib(C.CDLL(path), ref=True) if os.path.exists(path) else None
+    return _cache["r"]
