@@ -1,0 +1,243 @@
+"""Python host side of the MI355X-native fused Transform path.
+
+The product is the C++17 template library under include/fk/ (the operator API: PerThreadRead, .then(), Crop, Resize,
+Mul/Sub/Div, ColorConversion, TensorWrite, executeOperations) and its hand-written gfx950 kernels.  This module only
+loads the two native libraries built from it and exposes the chain entry points of include/fk_capi.h to Python, with
+torch tensors as device memory.  There is no CPU or eager fallback: if the native library is missing, or a call fails,
+an exception is raised.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+PRESERVE_AR, IGNORE_AR, PRESERVE_AR_RN_EVEN, PRESERVE_AR_LEFT = 0, 1, 2, 3
+BATCH_SIZES = (1, 2, 3, 5, 8, 32, 50)
+CHAIN_DEPTHS = (1, 2, 4, 8, 16, 32, 64, 128)
+
+
+class FkError(RuntimeError):
+    pass
+
+
+class Rect(C.Structure):
+    _fields_ = [("x", C.c_int), ("y", C.c_int), ("width", C.c_int), ("height", C.c_int)]
+
+
+def _rects(rects):
+    arr = (Rect * len(rects))()
+    for i, r in enumerate(rects):
+        arr[i] = Rect(*[int(v) for v in r])
+    return arr
+
+
+def _f3(v):
+    return (C.c_float * 3)(*[float(x) for x in v])
+
+
+_vp, _i, _f, _sz = C.c_void_p, C.c_int, C.c_float, C.c_size_t
+_f3p = C.POINTER(C.c_float)
+_rp = C.POINTER(Rect)
+
+CAPI_SIGNATURES = {
+    "fk_crop_resize_muls_bgr_tensor": [_vp, _i, _i, _sz, _rp, _i, _i, _i, _i, _f3p, _f3p, _f3p, _f3p, _vp, _vp],
+    "fk_muladd_chain_f32c3": [_vp, _i, _i, _sz, _i, _f, _f, _vp, _sz, _vp],
+    "fk_single_op_f32c3": [_vp, _i, _i, _sz, _i, _f, _vp, _sz, _vp],
+    "fk_batch_crop_resize_norm_split": [C.POINTER(C.c_void_p), _i, _i, _sz, _rp, _i, _i, _i, _f3p, _f3p, _f3p, _vp, _vp],
+    "fk_resize_crop_tiles": [_vp, _i, _i, _sz, _i, _i, _rp, _i, _i, _i, _f3p, _vp, _vp],
+    "fk_rgba2gray_u8c4": [_vp, _i, _i, _sz, _vp, _sz, _vp],
+    "fk_resize_mul_u8c4_f32c4": [_vp, _i, _i, _sz, _i, _i, _f, _vp, _sz, _vp],
+    "fk_crop_mul_saturate_u8c4": [_vp, _i, _i, _sz, Rect, _i, _vp, _sz, _vp],
+    "fk_rgba2bgr_sub_u8c4_f32c3": [_vp, _i, _i, _sz, _f, _vp, _sz, _vp],
+    "fk_divergent4_u8c4": [_vp, _i, _i, _sz, _vp, _i, _i, _f, _vp, Rect, _i, _vp, _f, _vp, _vp],
+    "fk_batch_crop_cast_tensor": [_vp, _i, _i, _sz, _rp, _i, _i, _i, _vp, _vp],
+}
+RUNTIME_SYMBOLS = [
+    "fkrt_device_count", "fkrt_set_device", "fkrt_get_device", "fkrt_stream_create", "fkrt_stream_destroy",
+    "fkrt_stream_sync", "fkrt_malloc", "fkrt_malloc_pitch", "fkrt_free", "fkrt_malloc_host", "fkrt_free_host",
+    "fkrt_memcpy_async", "fkrt_memcpy2d_async", "fkrt_memset_async", "fkrt_launch", "fkrt_params_upload",
+    "fkrt_params_release", "fkrt_max_kernarg_bytes", "fkrt_error_string", "fkrt_event_create", "fkrt_event_destroy",
+    "fkrt_event_record", "fkrt_event_sync", "fkrt_event_elapsed_ms",
+]
+
+_libs = {}
+
+
+def library_paths():
+    return os.path.join(_HERE, "libfk_hip_rt.so"), os.path.join(_HERE, "libfk_capi.so")
+
+
+def load():
+    """Load (once) and return (runtime, capi) ctypes handles; raises FkError when they have not been built."""
+    if "capi" not in _libs:
+        rt_path, capi_path = library_paths()
+        for p in (rt_path, capi_path):
+            if not os.path.exists(p):
+                raise FkError(f"native library {p} is missing: build it with `python -m fusedkernellibrary_amd.build`")
+        rt = C.CDLL(rt_path, mode=C.RTLD_GLOBAL)
+        capi = C.CDLL(capi_path)
+        for name, sig in CAPI_SIGNATURES.items():
+            fn = getattr(capi, name)
+            fn.argtypes = sig
+            fn.restype = C.c_int
+        capi.fk_last_error.restype = C.c_char_p
+        capi.fk_interpolate_y1_from_x.restype = C.c_int
+        rt.fkrt_error_string.restype = C.c_char_p
+        rt.fkrt_error_string.argtypes = [C.c_int]
+        rt.fkrt_max_kernarg_bytes.restype = C.c_size_t
+        rt.fkrt_event_create.argtypes = [C.POINTER(C.c_void_p)]
+        rt.fkrt_event_destroy.argtypes = [C.c_void_p]
+        rt.fkrt_event_record.argtypes = [C.c_void_p, C.c_void_p]
+        rt.fkrt_event_sync.argtypes = [C.c_void_p]
+        rt.fkrt_event_elapsed_ms.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        rt.fkrt_stream_create.argtypes = [C.POINTER(C.c_void_p)]
+        rt.fkrt_stream_destroy.argtypes = [C.c_void_p]
+        rt.fkrt_stream_sync.argtypes = [C.c_void_p]
+        _libs["rt"], _libs["capi"] = rt, capi
+    return _libs["rt"], _libs["capi"]
+
+
+def _check(rc):
+    if rc != 0:
+        _, capi = load()
+        kinds = {1: "unsupported", 2: "runtime", 3: "argument"}
+        raise FkError(f"fk call failed ({kinds.get(rc, rc)}): {capi.fk_last_error().decode()}")
+
+
+def _stream(stream):
+    if stream is not None:
+        return C.c_void_p(stream)
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(t, dtype_name):
+    import torch
+    if not t.is_cuda:
+        raise FkError("tensors must live on the GPU")
+    if t.dtype != getattr(torch, dtype_name):
+        raise FkError(f"expected a {dtype_name} tensor")
+    if t.stride(-1) != 1 or (t.dim() >= 3 and t.stride(-2) != t.shape[-1]):
+        raise FkError("pixels must be contiguous along a row")
+    return t
+
+
+def _image(t, dtype_name):
+    """(h, w, c) tensor whose row stride is the pitch -> (ptr, w, h, pitch_bytes)."""
+    t = _dev(t, dtype_name)
+    h, w = t.shape[0], t.shape[1]
+    return C.c_void_p(t.data_ptr()), w, h, t.stride(0) * t.element_size()
+
+
+# ---- chains: each mirrors one entry point of include/fk_capi.h; outputs are written into `out` ----------------------
+
+def crop_resize_muls_bgr_tensor(src, rects, out, aspect, background, mul, sub, div, stream=None):
+    """README pipeline. src: (H, W, 3) uint8; out: (n, dst_h, dst_w, 3) float32 contiguous."""
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    out = _dev(out, "float32")
+    n, dh, dw, _ = out.shape
+    assert n == len(rects) and out.is_contiguous()
+    _check(capi.fk_crop_resize_muls_bgr_tensor(p, w, h, pitch, _rects(rects), n, dw, dh, aspect, _f3(background), _f3(mul),
+                                               _f3(sub), _f3(div), C.c_void_p(out.data_ptr()), _stream(stream)))
+    return out
+
+
+def muladd_chain_f32c3(src, dst, depth, mul_v, add_v, stream=None):
+    _, capi = load()
+    p, w, h, pitch = _image(src, "float32")
+    q, w2, h2, pitch2 = _image(dst, "float32")
+    assert (w, h) == (w2, h2)
+    _check(capi.fk_muladd_chain_f32c3(p, w, h, pitch, depth, mul_v, add_v, q, pitch2, _stream(stream)))
+    return dst
+
+
+def single_op_f32c3(src, dst, is_add, v, stream=None):
+    _, capi = load()
+    p, w, h, pitch = _image(src, "float32")
+    q, w2, h2, pitch2 = _image(dst, "float32")
+    assert (w, h) == (w2, h2)
+    _check(capi.fk_single_op_f32c3(p, w, h, pitch, int(is_add), v, q, pitch2, _stream(stream)))
+    return dst
+
+
+def batch_crop_resize_norm_split(srcs, rects, out, div1, sub, div2, stream=None):
+    """srcs: list of (H, W, 3) uint8 of one size/pitch; out: (n, 3, dst_h, dst_w) float32 contiguous."""
+    _, capi = load()
+    n = len(srcs)
+    p0, w, h, pitch = _image(srcs[0], "uint8")
+    for s in srcs:
+        assert _image(s, "uint8")[1:] == (w, h, pitch)
+    ptrs = (C.c_void_p * n)(*[s.data_ptr() for s in srcs])
+    out = _dev(out, "float32")
+    assert out.shape[0] == n == len(rects) and out.shape[1] == 3 and out.is_contiguous()
+    _check(capi.fk_batch_crop_resize_norm_split(ptrs, w, h, pitch, _rects(rects), n, out.shape[3], out.shape[2], _f3(div1),
+                                                _f3(sub), _f3(div2), C.c_void_p(out.data_ptr()), _stream(stream)))
+    return out
+
+
+def resize_crop_tiles(src, resized, rects, out, mul, stream=None):
+    """src: (H, W, 3) uint8; resized = (rs_w, rs_h); out: (n, tile_h, tile_w, 3) float32 contiguous."""
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    out = _dev(out, "float32")
+    n, th, tw, _ = out.shape
+    assert n == len(rects) and out.is_contiguous()
+    _check(capi.fk_resize_crop_tiles(p, w, h, pitch, resized[0], resized[1], _rects(rects), n, tw, th, _f3(mul),
+                                     C.c_void_p(out.data_ptr()), _stream(stream)))
+    return out
+
+
+def rgba2gray_u8c4(src, dst, stream=None):
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    d = _dev(dst, "uint8")
+    _check(capi.fk_rgba2gray_u8c4(p, w, h, pitch, C.c_void_p(d.data_ptr()), d.stride(0), _stream(stream)))
+    return dst
+
+
+def resize_mul_u8c4_f32c4(src, dst, mul_v, stream=None):
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    q, dw, dh, dpitch = _image(dst, "float32")
+    _check(capi.fk_resize_mul_u8c4_f32c4(p, w, h, pitch, dw, dh, mul_v, q, dpitch, _stream(stream)))
+    return dst
+
+
+def crop_mul_saturate_u8c4(src, rect, dst, mul_v, stream=None):
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    q, _, _, dpitch = _image(dst, "uint8")
+    _check(capi.fk_crop_mul_saturate_u8c4(p, w, h, pitch, Rect(*rect), mul_v, q, dpitch, _stream(stream)))
+    return dst
+
+
+def rgba2bgr_sub_u8c4_f32c3(src, dst, sub_v, stream=None):
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    q, _, _, dpitch = _image(dst, "float32")
+    _check(capi.fk_rgba2bgr_sub_u8c4_f32c3(p, w, h, pitch, sub_v, q, dpitch, _stream(stream)))
+    return dst
+
+
+def divergent4_u8c4(src, gray_out, resized_out, mul_b, rect_c, mul_c, crop_out, sub_d, bgr_out, stream=None):
+    """All four chains in one launch; outputs must be contiguous."""
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    for t in (gray_out, resized_out, crop_out, bgr_out):
+        assert t.is_contiguous()
+    _check(capi.fk_divergent4_u8c4(p, w, h, pitch, C.c_void_p(_dev(gray_out, "uint8").data_ptr()), resized_out.shape[1],
+                                   resized_out.shape[0], mul_b, C.c_void_p(_dev(resized_out, "float32").data_ptr()),
+                                   Rect(*rect_c), mul_c, C.c_void_p(_dev(crop_out, "uint8").data_ptr()), sub_d,
+                                   C.c_void_p(_dev(bgr_out, "float32").data_ptr()), _stream(stream)))
+
+
+def batch_crop_cast_tensor(src, rects, out, stream=None):
+    """out: (n, max_h, max_w, 3) float32 contiguous; elements outside a plane's own rect stay untouched."""
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    out = _dev(out, "float32")
+    n, mh, mw, _ = out.shape
+    assert n == len(rects) and out.is_contiguous()
+    _check(capi.fk_batch_crop_cast_tensor(p, w, h, pitch, _rects(rects), n, mw, mh, C.c_void_p(out.data_ptr()), _stream(stream)))
+    return out

@@ -1,0 +1,61 @@
+"""Build recipe of the native libraries (hipcc, gfx950 only).
+
+  libfk_hip_rt.so   the C runtime ABI of include/fk_hip_rt.h (csrc/fk_hip_rt.cpp)
+  libfk_capi.so     the chain entry points of include/fk_capi.h (csrc/fk_capi.hip), i.e. the fused kernels
+                    instantiated from the fk:: templates under include/fk/
+
+Run as `python -m fusedkernellibrary_amd.build`; outputs land beside this file.
+"""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+INCLUDE = os.path.join(ROOT, "include")
+CSRC = os.path.join(HERE, "csrc")
+
+# -ffp-contract=off: no FMA contraction, so results equal an unfused evaluation bit for bit.
+# packed-fp32-ops is switched off for device code (the host pass warns that it does not know the feature).
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-std=c++17", "-O3", "-ffp-contract=off", "-ftemplate-depth=1024",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def hipcc():
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: the native libraries cannot be built")
+    return exe
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stdout)
+        raise RuntimeError("build step failed: " + " ".join(cmd))
+    return proc.stdout
+
+
+def build_runtime():
+    out = os.path.join(HERE, "libfk_hip_rt.so")
+    _run([hipcc(), os.path.join(CSRC, "fk_hip_rt.cpp"), "-I" + INCLUDE, "-std=c++17", "-O2", "-fPIC", "-shared", "-o", out])
+    return out
+
+
+def build_capi(extra_defines=(), name="libfk_capi.so"):
+    out = os.path.join(HERE, name)
+    cmd = [hipcc(), "-x", "hip", os.path.join(CSRC, "fk_capi.hip"), "-I" + INCLUDE, *DEVICE_FLAGS, "-fPIC", "-shared",
+           "-L" + HERE, "-lfk_hip_rt", "-Wl,-rpath,$ORIGIN", "-o", out]
+    cmd += ["-D" + d for d in extra_defines]
+    _run(cmd)
+    return out
+
+
+def build_all():
+    return [build_runtime(), build_capi()]
+
+
+if __name__ == "__main__":
+    for path in build_all():
+        print(path)

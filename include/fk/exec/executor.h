@@ -1,0 +1,297 @@
+// Host dispatch: TransformDPP / DivergentBatchTransformDPP tags, Executor and job construction.
+//
+// API counterpart of the reference's core/execution_model/data_parallel_patterns.h:65-67,194-235,301-353 (the DPP
+// types named in executeOperations<...>) and core/execution_model/executors.h:44-128,245-293 (Executor, the overload
+// set of executeOperations, grid computation and launch).  A chain is analysed at compile time into one of the
+// kernel families of fk/exec/kernels.h; the launch itself goes through the C runtime ABI (fkrt_launch).
+#ifndef FK_EXEC_EXECUTOR_H
+#define FK_EXEC_EXECUTOR_H
+
+#include <cstring>
+#include <tuple>
+#include <memory>
+
+#include "fk/core/stream.h"
+#include "fk/exec/kernels.h"
+
+namespace fk {
+
+template <ParArch PA = defaultParArch, TF TFEN = TF::DISABLED>
+struct TransformDPP {
+    static constexpr ParArch PAR_ARCH = PA;
+    static_assert(PA == ParArch::GPU_AMD,
+                  "Only ParArch::GPU_AMD is implemented by this library; there is no host fallback executor.");
+};
+
+// One fused chain per group of thread planes, all in one launch.
+template <ParArch PA = defaultParArch>
+struct DivergentBatchTransformDPP {
+    static constexpr ParArch PAR_ARCH = PA;
+    static_assert(PA == ParArch::GPU_AMD,
+                  "Only ParArch::GPU_AMD is implemented by this library; there is no host fallback executor.");
+};
+
+// A (sender..., receiver) chain kept as a value, for divergent launches (core/data/tuple.h:199-215).
+template <typename Sender, typename Receiver>
+struct InstantiableOperationSequence {
+    Sender sender;
+    Receiver receiver;
+};
+template <typename First, typename... Rest>
+inline constexpr auto buildOperationSequence(const First& first, const Rest&... rest);
+
+namespace exec {
+
+inline unsigned ceil_div(unsigned a, unsigned b) { return (a + b - 1u) / b; }
+inline bool aligned_to(const void* p, size_t a) { return reinterpret_cast<size_t>(p) % a == 0; }
+
+// ---- job construction ----------------------------------------------------------------------------------------
+namespace detail {
+template <typename Sender, typename = void>
+struct PlaneIOpOf {
+    using type = Sender;
+    static constexpr size_t planes = 1;
+    static constexpr bool process_all = true;
+    static const type& get(const Sender& s, size_t) { return s; }
+};
+template <typename Sender>
+struct PlaneIOpOf<Sender, std::enable_if_t<isBatchOperation<typename Sender::Operation>>> {
+    using Batch = typename Sender::Operation;
+    using type = Instantiable<typename Batch::Operation>;
+    static constexpr size_t planes = Batch::BATCH;
+    static constexpr bool process_all = Batch::PP == PlanePolicy::PROCESS_ALL;
+    static type get(const Sender& s, size_t i) { return toIOp<typename Batch::Operation>(s.params.opData[i]); }
+};
+template <typename PlaneIOp, typename Receiver, typename = void>
+struct Matches : std::false_type {};
+template <typename PlaneIOp, typename Receiver>
+struct Matches<PlaneIOp, Receiver, std::enable_if_t<ProgramOf<PlaneIOp>::supported && OutOf<Receiver>::supported>>
+    : std::is_same<typename ProgramOf<PlaneIOp>::OutputType, typename OutOf<Receiver>::type::Pixel> {};
+} // namespace detail
+
+template <typename Sender, typename Receiver>
+struct JobOf {
+    using Planes = detail::PlaneIOpOf<Sender>;
+    using PlaneIOp = typename Planes::type;
+    static constexpr size_t N = Planes::planes;
+    static constexpr bool viewable = Planes::process_all && detail::Matches<PlaneIOp, Receiver>::value;
+
+    static auto make(const Sender& sender, const Receiver& receiver) {
+        if constexpr (viewable) {
+            using Prog = typename ProgramOf<PlaneIOp>::type;
+            using Out = typename OutOf<Receiver>::type;
+            using View = decltype(Prog::view);
+            const Out out = OutOf<Receiver>::make(receiver);
+            if constexpr (View::IS_RESIZE) {
+                ResizeJob<Prog, N, Out> job{};
+                int max_w = 0, max_h = 0;
+                for (size_t i = 0; i < N; ++i) {
+                    job.plane[i] = ProgramOf<PlaneIOp>::make(Planes::get(sender, i));
+                    max_w = job.plane[i].view.w > max_w ? job.plane[i].view.w : max_w;
+                    max_h = job.plane[i].view.h > max_h ? job.plane[i].view.h : max_h;
+                }
+                job.out = out;
+                job.grid_x = ceil_div(static_cast<unsigned>(max_w), RESIZE_TILE_W);
+                job.grid_y = ceil_div(static_cast<unsigned>(max_h), RESIZE_TILE_H);
+                return job;
+            } else {
+                using Job = PointwiseJob<Prog, N, Out>;
+                using Src = typename Job::Src;
+                Job job{};
+                job.out = out;
+                constexpr size_t in_chunk = dev::chunk_bytes(Job::K * static_cast<int>(sizeof(Src)));
+                constexpr size_t out_elem = Out::IS_SPLIT ? sizeof(VBase<typename Out::Pixel>) : sizeof(typename Out::Pixel);
+                constexpr size_t out_chunk = dev::chunk_bytes(Job::K * static_cast<int>(out_elem));
+                int max_w = 0, max_h = 0;
+                for (size_t i = 0; i < N; ++i) {
+                    job.plane[i].prog = ProgramOf<PlaneIOp>::make(Planes::get(sender, i));
+                    auto& v = job.plane[i].prog.view;
+                    if (N == 1 && v.ox == 0 && v.oy == 0 && v.w == v.img_w && v.h > 1 &&
+                        v.pitch == static_cast<uint>(v.w) * sizeof(Src) && out.pitch == static_cast<uint>(v.w) * out_elem &&
+                        static_cast<size_t>(v.w) * v.h < (1u << 30)) {
+                        // rows are contiguous on both sides: treat the image as one long row, so no block is cut
+                        // short at a row end
+                        v.w = v.img_w = v.w * v.h;
+                        v.h = v.img_h = 1;
+                    }
+                    const char* const first = reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy) * v.pitch +
+                                              static_cast<size_t>(v.ox) * sizeof(Src);
+                    bool vec = aligned_to(first, in_chunk) && (v.h == 1 || v.pitch % in_chunk == 0);
+                    const char* const ofirst = reinterpret_cast<const char*>(out.data) + i * out.z_stride;
+                    vec = vec && aligned_to(ofirst, out_chunk) && (v.h == 1 || out.pitch % out_chunk == 0);
+                    if constexpr (Out::IS_SPLIT) vec = vec && out.chan_stride % out_chunk == 0;
+                    job.plane[i].flags = vec ? FLAG_VECTOR_IO : 0u;
+                    max_w = v.w > max_w ? v.w : max_w;
+                    max_h = v.h > max_h ? v.h : max_h;
+                }
+                // thread columns per block: enough to span the widest row, at most the whole block
+                const unsigned groups = ceil_div(static_cast<unsigned>(max_w), Job::K);
+                unsigned shift = 0;
+                while ((1u << shift) < groups && shift < 8u) ++shift;
+                if (shift < 4u) shift = 4u; // keep a wave's accesses within a few rows
+                job.tx_shift = shift;
+                job.grid_x = ceil_div(groups, 1u << shift);
+                job.grid_y = ceil_div(static_cast<unsigned>(max_h), BLOCK_THREADS >> shift);
+                return job;
+            }
+        } else {
+            GenericJob<Sender, Receiver> job{};
+            job.sender = sender;
+            job.receiver = receiver;
+            job.active = sender.getActiveThreads();
+            job.grid_x = ceil_div(job.active.x, 64u);
+            job.grid_y = ceil_div(job.active.y, 4u);
+            return job;
+        }
+    }
+    static unsigned planes(const Sender& sender) {
+        if constexpr (viewable) return static_cast<unsigned>(N);
+        else return sender.getActiveThreads().z;
+    }
+};
+
+// Launch `kernel(args)` by value, or through a staged copy when `Args` exceeds the kernel-argument limit.
+template <typename Args>
+inline void launch_args(const void* by_value, const void* indirect, const Args& args, unsigned gx, unsigned gy, unsigned gz,
+                        size_t lds_bytes, fkrt_stream stream) {
+    if (gx == 0 || gy == 0 || gz == 0) return; // nothing to do
+    if (sizeof(Args) <= fkrt_max_kernarg_bytes()) {
+        void* argv[] = { const_cast<Args*>(&args) };
+        gpuErrchk(fkrt_launch(by_value, gx, gy, gz, BLOCK_THREADS, 1, 1, argv, lds_bytes, stream));
+    } else {
+        void* device_args = nullptr;
+        gpuErrchk(fkrt_params_upload(&device_args, &args, sizeof(Args), stream));
+        void* argv[] = { &device_args };
+        const int status = fkrt_launch(indirect, gx, gy, gz, BLOCK_THREADS, 1, 1, argv, lds_bytes, stream);
+        gpuErrchk(fkrt_params_release(device_args, stream));
+        gpuErrchk(status);
+    }
+}
+
+template <typename Job>
+inline void launch_job(const Job& job, unsigned planes, fkrt_stream stream) {
+    launch_args(reinterpret_cast<const void*>(&transform_kernel<Job>), reinterpret_cast<const void*>(&transform_kernel_indirect<Job>),
+                job, job.grid_x, job.grid_y, planes, Job::LDS_BYTES, stream);
+}
+
+// (read, compute..., write) as (sender, receiver)
+template <typename Receiver>
+inline constexpr const Receiver& last_of(const Receiver& r) { return r; }
+template <typename First, typename... Rest>
+inline constexpr const auto& last_of(const First&, const Rest&... rest) { return last_of(rest...); }
+
+template <size_t... Idx, typename Tuple>
+inline constexpr auto fuse_front(std::index_sequence<Idx...>, const Tuple& t) {
+    if constexpr (sizeof...(Idx) == 1) {
+        return std::get<0>(t);
+    } else {
+        return Fuser::fuse(std::get<Idx>(t)...);
+    }
+}
+template <typename... IOps>
+inline constexpr auto sender_of(const IOps&... iOps) {
+    static_assert(sizeof...(IOps) >= 2, "A chain needs at least a read and a write operation.");
+    return fuse_front(std::make_index_sequence<sizeof...(IOps) - 1>{}, std::forward_as_tuple(iOps...));
+}
+
+} // namespace exec
+
+template <typename First, typename... Rest>
+inline constexpr auto buildOperationSequence(const First& first, const Rest&... rest) {
+    const auto sender = exec::sender_of(first, rest...);
+    const auto& receiver = exec::last_of(rest...);
+    static_assert(isAnyReadType<std::decay_t<decltype(sender)>>, "The first operation of a chain must be a read.");
+    static_assert(isWriteType<std::decay_t<decltype(receiver)>>, "The last operation of a chain must be a write.");
+    return InstantiableOperationSequence<std::decay_t<decltype(sender)>, std::decay_t<decltype(receiver)>>{ sender, receiver };
+}
+
+template <typename DPP>
+struct Executor;
+
+template <TF TFEN>
+struct Executor<TransformDPP<ParArch::GPU_AMD, TFEN>> {
+    FK_STATIC_STRUCT(Executor, Executor)
+    static constexpr ParArch parArch() { return ParArch::GPU_AMD; }
+
+    // executeOperations(stream, read, [compute...], write): one kernel for the whole chain
+    template <typename... IOps>
+    static inline void executeOperations(Stream_<ParArch::GPU_AMD>& stream, const IOps&... iOps) {
+        const auto seq = buildOperationSequence(iOps...);
+        using Sender = std::decay_t<decltype(seq.sender)>;
+        using Receiver = std::decay_t<decltype(seq.receiver)>;
+        using Plan = exec::JobOf<Sender, Receiver>;
+        const auto job = Plan::make(seq.sender, seq.receiver);
+        exec::launch_job(job, Plan::planes(seq.sender), stream.getHIPStream());
+    }
+    // Convenience forms over buffers (executors.h:52-93).
+    template <ND D, typename I, typename... IOps>
+    static inline void executeOperations(const Ptr<D, I>& input, Stream_<ParArch::GPU_AMD>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<D, I>::build(input), iOps...);
+    }
+    template <ND D, typename I, typename O, typename... IOps>
+    static inline void executeOperations(const Ptr<D, I>& input, const Ptr<D, O>& output, Stream_<ParArch::GPU_AMD>& stream,
+                                         const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<D, I>::build(input), iOps..., PerThreadWrite<D, O>::build(output));
+    }
+    template <typename I, size_t BATCH, typename... IOps>
+    static inline void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, const int& activeBatch, const I& defaultValue,
+                                         Stream_<ParArch::GPU_AMD>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<ND::_2D, I>::build(activeBatch, defaultValue, input), iOps...);
+    }
+    template <typename I, size_t BATCH, typename... IOps>
+    static inline void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, Stream_<ParArch::GPU_AMD>& stream,
+                                         const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<ND::_2D, I>::build(input), iOps...);
+    }
+    template <typename I, typename O, size_t BATCH, typename... IOps>
+    static inline void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, const int& activeBatch, const I& defaultValue,
+                                         const Tensor<O>& output, Stream_<ParArch::GPU_AMD>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<ND::_2D, I>::build(activeBatch, defaultValue, input), iOps...,
+                          PerThreadWrite<ND::_3D, O>::build(output));
+    }
+    template <typename I, typename O, size_t BATCH, typename... IOps>
+    static inline void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, const Tensor<O>& output,
+                                         Stream_<ParArch::GPU_AMD>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<ND::_2D, I>::build(input), iOps..., PerThreadWrite<ND::_3D, O>::build(output));
+    }
+};
+
+template <>
+struct Executor<DivergentBatchTransformDPP<ParArch::GPU_AMD>> {
+    FK_STATIC_STRUCT(Executor, Executor)
+    static constexpr ParArch parArch() { return ParArch::GPU_AMD; }
+
+    // executeOperations(stream, sequence0, sequence1, ...): every sequence is a chain built with
+    // buildOperationSequence; all of them run in one launch, each over its own planes.
+    template <typename... Senders, typename... Receivers>
+    static inline void executeOperations(Stream_<ParArch::GPU_AMD>& stream,
+                                         const InstantiableOperationSequence<Senders, Receivers>&... sequences) {
+        static_assert(sizeof...(Senders) >= 1, "A divergent launch needs at least one sequence.");
+        using Pack = exec::JobPack<std::decay_t<decltype(exec::JobOf<Senders, Receivers>::make(sequences.sender, sequences.receiver))>...>;
+        // the pack holds every job by value; build it on the heap, it can be several KiB
+        auto pack = std::make_unique<Pack>();
+        unsigned total = 0;
+        size_t lds = 0;
+        fill(*pack, total, lds, sequences...);
+        exec::launch_args(reinterpret_cast<const void*>(&exec::divergent_kernel<Pack>),
+                          reinterpret_cast<const void*>(&exec::divergent_kernel_indirect<Pack>), *pack, total, 1, 1, lds,
+                          stream.getHIPStream());
+    }
+
+private:
+    template <typename Pack>
+    static inline void fill(Pack&, unsigned&, size_t&) {}
+    template <typename Pack, typename Seq, typename... Rest>
+    static inline void fill(Pack& pack, unsigned& total, size_t& lds, const Seq& seq, const Rest&... rest) {
+        using Plan = exec::JobOf<std::decay_t<decltype(seq.sender)>, std::decay_t<decltype(seq.receiver)>>;
+        pack.job = Plan::make(seq.sender, seq.receiver);
+        pack.blocks = pack.job.grid_x * pack.job.grid_y * Plan::planes(seq.sender);
+        total += pack.blocks;
+        using Job = std::decay_t<decltype(pack.job)>;
+        lds = lds > static_cast<size_t>(Job::LDS_BYTES) ? lds : static_cast<size_t>(Job::LDS_BYTES);
+        fill(pack.rest, total, lds, rest...);
+    }
+};
+
+} // namespace fk
+#endif

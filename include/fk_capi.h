@@ -1,0 +1,94 @@
+/* fk_capi.h — C entry points for the fused chains of the Transform data-parallel path.
+ *
+ * The reference has no FFI: its operator API is C++17 templates, so a chain is fixed at compile time.  Each function
+ * below is one such chain, instantiated from this library's fk:: templates (include/fk/) for a caller that cannot
+ * compile templates (ctypes, cgo, JNI ...).  Device pointers and sizes only; `stream` is a hipStream_t (NULL = default
+ * stream); work is enqueued asynchronously, the caller synchronises the stream.  Return value: 0 = enqueued,
+ * FK_ERR_UNSUPPORTED = the batch size / depth / mode has no instantiation, FK_ERR_RUNTIME = the GPU runtime reported
+ * an error (text from fk_last_error()), FK_ERR_ARGUMENT = inconsistent arguments.
+ *
+ * Reference interface each one stands for (paths below the reference's include/fused_kernel/ unless noted):
+ *   every function: executeOperations<TransformDPP<>>(stream, sender, receiver), fused_kernel.h:22-25, with the chain
+ *   built by .then() (core/execution_model/operation_model/instantiable_operations.h:44-52).
+ */
+#ifndef FK_CAPI_H
+#define FK_CAPI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { FK_OK = 0, FK_ERR_UNSUPPORTED = 1, FK_ERR_RUNTIME = 2, FK_ERR_ARGUMENT = 3 };
+
+/* Rect_<uint,int>, core/data/rect.h:23-32 */
+typedef struct fk_rect {
+    int x, y, width, height;
+} fk_rect;
+
+/* AspectRatio, algorithms/image_processing/resize.h:42 */
+enum { FK_PRESERVE_AR = 0, FK_IGNORE_AR = 1, FK_PRESERVE_AR_RN_EVEN = 2, FK_PRESERVE_AR_LEFT = 3 };
+
+const char* fk_last_error(void);
+/* 0 when the library was built with the bilinear row index taken from y (the reference's device branch,
+ * algorithms/image_processing/interpolation.h:66-67); 1 for a build that takes it from x (its host branch, :69-70). */
+int fk_interpolate_y1_from_x(void);
+
+/* The README pipeline (tests/examples/readme_test_code.h:26-72 of the reference):
+ * PerThreadRead<_2D,uchar3> -> Crop(rects[n]) -> Resize<INTER_LINEAR, aspect>(dst_w x dst_h, background) ->
+ * Mul<float3> -> Sub<float3> -> Div<float3> -> ColorConversion<COLOR_RGB2BGR> -> TensorWrite<float3>.
+ * out: n planes of dst_h x dst_w packed float3.  n in {1,2,3,5,8,32,50}. */
+int fk_crop_resize_muls_bgr_tensor(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n,
+                                   int dst_w, int dst_h, int aspect, const float background[3], const float mul[3],
+                                   const float sub[3], const float div[3], float* out, void* stream);
+
+/* Vertical fusion: PerThreadRead<_2D,float3> -> depth x alternating Mul<float3>(mul_v) / Add<float3>(add_v)
+ * (operation 0 is Mul) -> PerThreadWrite<_2D,float3>, one launch.  depth in {1,2,4,8,16,32,64,128}.
+ * (algorithms/basic_ops/arithmetic.h:22-88; benchmarks/numinstructions/benchmark_numinstructions_x_operation.h:68-99
+ * of the reference builds the same kind of chain.) */
+int fk_muladd_chain_f32c3(const void* src, int w, int h, size_t src_pitch, int depth, float mul_v, float add_v, void* dst,
+                          size_t dst_pitch, void* stream);
+/* One unfused stage of that chain: read -> Mul or Add -> write. */
+int fk_single_op_f32c3(const void* src, int w, int h, size_t src_pitch, int is_add, float v, void* dst, size_t dst_pitch,
+                       void* stream);
+
+/* Horizontal fusion: PerThreadRead(array of n images) -> Crop(rects[n]) -> Resize<INTER_LINEAR>(dst) -> Div<float3> ->
+ * Sub<float3> -> Div<float3> -> COLOR_RGB2BGR -> TensorSplit<float3> (memory_operations.h:195-226).
+ * srcs: host array of n device pointers.  out: n x 3 x dst_h x dst_w planar float.  n in {1,2,3,5,8,32,50}. */
+int fk_batch_crop_resize_norm_split(const void* const* srcs, int src_w, int src_h, size_t src_pitch, const fk_rect* rects,
+                                    int n, int dst_w, int dst_h, const float div1[3], const float sub[3],
+                                    const float div2[3], float* out, void* stream);
+
+/* Backwards vertical fusion: PerThreadRead<_2D,uchar3> -> Resize<INTER_LINEAR>(rs_w x rs_h) -> Crop(rects[n]) ->
+ * Mul<float3> -> TensorWrite<float3>; no resized image is materialised.  out: n x tile_h x tile_w float3. */
+int fk_resize_crop_tiles(const void* src, int src_w, int src_h, size_t src_pitch, int rs_w, int rs_h, const fk_rect* rects,
+                         int n, int tile_w, int tile_h, const float mul[3], float* out, void* stream);
+
+/* The four chains of the divergent launch, runnable on their own ... */
+int fk_rgba2gray_u8c4(const void* src, int w, int h, size_t src_pitch, void* dst, size_t dst_pitch, void* stream);
+int fk_resize_mul_u8c4_f32c4(const void* src, int w, int h, size_t src_pitch, int dst_w, int dst_h, float mul_v, void* dst,
+                             size_t dst_pitch, void* stream);
+int fk_crop_mul_saturate_u8c4(const void* src, int w, int h, size_t src_pitch, fk_rect rect, int mul_v, void* dst,
+                              size_t dst_pitch, void* stream);
+int fk_rgba2bgr_sub_u8c4_f32c3(const void* src, int w, int h, size_t src_pitch, float sub_v, void* dst, size_t dst_pitch,
+                               void* stream);
+/* ... and as ONE launch (executeOperations<DivergentBatchTransformDPP<>>; the reference declares the pattern in
+ * core/execution_model/data_parallel_patterns.h:301-353 but ships no executor for it):
+ * (a) COLOR_RGBA2GRAY -> uchar; (b) Resize<INTER_LINEAR>(rs_w x rs_h) -> Mul<float4>(mul_b) -> float4;
+ * (c) Crop(rect_c) -> Mul<uchar4,int,int4>(mul_c) -> SaturateCast<int4,uchar4>; (d) COLOR_RGBA2BGR -> Cast<float3> ->
+ * Sub<float3>(sub_d).  Output rows are tight. */
+int fk_divergent4_u8c4(const void* src, int w, int h, size_t src_pitch, void* gray_out, int rs_w, int rs_h, float mul_b,
+                       void* resized_out, fk_rect rect_c, int mul_c, void* crop_out, float sub_d, void* bgr_out,
+                       void* stream);
+
+/* Ragged batch without resize: PerThreadRead -> Crop(rects[n]) -> Cast<uchar3,float3> -> TensorWrite<float3> into a
+ * max_w x max_h x n tensor.  Elements outside a plane's own rect are left untouched. */
+int fk_batch_crop_cast_tensor(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n,
+                              int max_w, int max_h, float* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

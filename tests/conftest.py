@@ -1,0 +1,45 @@
+import os
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs an MI355X; run on the GPU box only")
+
+
+@pytest.fixture(scope="session")
+def oracle():
+    from oracle import binding
+    return binding.oracle()
+
+
+@pytest.fixture(scope="session")
+def reference():
+    """The reference-headers build (literal host semantics); tests that need it skip when it was not built."""
+    from oracle import binding
+    ref = binding.reference()
+    if ref is None:
+        pytest.skip("oracle/_ref/libfkref.so not built (needs the reference tree)")
+    return ref
+
+
+@pytest.fixture(scope="session")
+def fk():
+    """The native library on the GPU.  Never falls back: a missing library is an error, not a skip."""
+    import torch
+    import fusedkernellibrary_amd as lib
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    lib.load()
+    return lib
+
+
+def same_bits(a, b):
+    a = np.ascontiguousarray(a)
+    b = np.ascontiguousarray(b)
+    return a.shape == b.shape and a.dtype == b.dtype and a.tobytes() == b.tobytes()
