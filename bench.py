@@ -1,0 +1,229 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused Transform path on one MI355X.
+
+Headline workload (BASELINE.json configs[1]): 3840x2160 float3, PerThreadRead -> 16 alternating Mul/Add ->
+PerThreadWrite in ONE launch.  One step = one fused launch over the whole image.  Inputs are resident in HBM before
+the timed region; three buffer sets (600 MB) are rotated so that the 256 MB Infinity Cache cannot hold a step's data.
+Prints ONE JSON line: Gpixel/s, the HBM roofline of the kernel (algorithmic bytes / measured duration vs 8 TB/s),
+the reference CPU executor timed on this host, and per-config figures for the other chains.
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12
+W, H = 3840, 2160
+DEPTH = 16
+MUL_V, ADD_V = 1.0001, 1e-4
+
+
+class StreamTimer:
+    """HIP events on the stream the kernels are launched on (through the library's own runtime ABI)."""
+
+    def __init__(self, rt, stream):
+        self.rt, self.stream = rt, C.c_void_p(stream)
+        self.a, self.b = C.c_void_p(), C.c_void_p()
+        assert rt.fkrt_event_create(C.byref(self.a)) == 0 and rt.fkrt_event_create(C.byref(self.b)) == 0
+
+    def start(self):
+        assert self.rt.fkrt_event_record(self.a, self.stream) == 0
+
+    def stop_ms(self):
+        assert self.rt.fkrt_event_record(self.b, self.stream) == 0
+        assert self.rt.fkrt_event_sync(self.b) == 0
+        ms = C.c_float()
+        assert self.rt.fkrt_event_elapsed_ms(C.byref(ms), self.a, self.b) == 0
+        return float(ms.value)
+
+
+def time_launches(timer, launch, steps, warmup):
+    import torch
+    for i in range(warmup):
+        launch(i)
+    torch.cuda.synchronize()
+    timer.start()
+    for i in range(steps):
+        launch(i)
+    ms = timer.stop_ms()
+    torch.cuda.synchronize()
+    return ms / steps
+
+
+def cpu_baseline(src_host, budget_s=10.0):
+    """The reference's own CPU executor (oracle/_ref, its headers compiled as they are) on the same chain and image,
+    one core; falls back to the C restatement when that build is absent."""
+    import numpy as np
+    from oracle import binding
+    ref = binding.reference()
+    lib, kind = (ref, "reference") if ref is not None else (binding.oracle(), "port")
+    lib.muladd_chain_f32c3(src_host[:64], DEPTH, MUL_V, ADD_V)  # warm-up
+    passes, t0 = 0, time.perf_counter()
+    while True:
+        lib.muladd_chain_f32c3(src_host, DEPTH, MUL_V, ADD_V)
+        passes += 1
+        dt = time.perf_counter() - t0
+        if dt >= budget_s or passes >= 200:
+            break
+    return {"value": W * H * passes / dt / 1e9, "unit": "Gpixel/s", "cores": 1, "kind": kind,
+            "sample": f"{passes} full passes of the same {W}x{H} float3 depth-{DEPTH} chain in {dt:.1f} s, serial z/y/x loop",
+            "ms_per_pass": 1e3 * dt / passes, "host_cores_available": os.cpu_count()}
+
+
+def other_configs(fk, timer, steps, warmup):
+    """Per-config kernel time, output Gpixel/s and algorithmic GB/s for the remaining chains (device-random inputs)."""
+    import torch
+    res = {}
+    g = torch.Generator(device="cuda").manual_seed(0)
+
+    def rnd_u8(*shape):
+        return torch.randint(0, 256, shape, dtype=torch.uint8, device="cuda", generator=g)
+
+    def record(name, ms, out_px, alg_bytes, note=None):
+        res[name] = {"ms": ms, "gpixel_s": out_px / ms / 1e6, "alg_bytes": alg_bytes, "gb_s": alg_bytes / ms / 1e6,
+                     "frac_hbm_peak": alg_bytes / (ms * 1e-3) / HBM_PEAK}
+        if note:
+            res[name]["note"] = note
+
+    # C1: README pipeline at its literal shape (launch-latency bound: 234 KB moved)
+    img4k = rnd_u8(2160, 3840, 3)
+    rects = [(0, 0, 34, 25), (10, 10, 70, 15), (20, 20, 60, 59), (30, 30, 20, 23), (40, 40, 12, 11)]
+    out1 = torch.empty((5, 60, 60, 3), device="cuda")
+    a1 = (0, (0, 0, 0), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)
+    ms = time_launches(timer, lambda i: fk.crop_resize_muls_bgr_tensor(img4k, rects, out1, *a1), steps, warmup)
+    record("C1_readme_60x60x5", ms, 18000, sum(r[2] * r[3] for r in rects) * 3 + 18000 * 12, "launch-latency bound")
+
+    # C1 scaled: same chain, 5 crops of 1024x768 -> 1920x1080 (bandwidth-sized)
+    rects_s = [(64 * i, 48 * i, 1024, 768) for i in range(5)]
+    out1s = [torch.empty((5, 1080, 1920, 3), device="cuda") for _ in range(3)]
+    ms = time_launches(timer, lambda i: fk.crop_resize_muls_bgr_tensor(img4k, rects_s, out1s[i % 3], *a1), steps, warmup)
+    record("C1_scaled_5x1024x768_to_1920x1080", ms, 5 * 1920 * 1080, 5 * 1024 * 768 * 3 + 5 * 1920 * 1080 * 12)
+
+    # C3: 50 crops of 50 images -> 224x224x3x50 planar
+    imgs = [rnd_u8(1080, 1920, 3) for _ in range(50)]
+    ws = torch.randint(16, 513, (50,), generator=torch.Generator().manual_seed(3)).tolist()
+    hs = torch.randint(16, 513, (50,), generator=torch.Generator().manual_seed(4)).tolist()
+    rects3 = [((1920 - w) // 2, (1080 - h) // 3, w, h) for w, h in zip(ws, hs)]
+    out3 = torch.empty((50, 3, 224, 224), device="cuda")
+    a3 = ((255.,) * 3, (.485, .456, .406), (.229, .224, .225))
+    ms = time_launches(timer, lambda i: fk.batch_crop_resize_norm_split(imgs, rects3, out3, *a3), steps, warmup)
+    record("C3_batch50_224x224_split", ms, 50 * 224 * 224, 50 * 224 * 224 * 12 + sum(3 * r[2] * r[3] for r in rects3))
+    del imgs
+
+    # C4: resize 4K -> 1280x720, 32 tiles of 128x128
+    rects4 = [(160 * i, 180 * j, 128, 128) for j in range(4) for i in range(8)]
+    out4 = torch.empty((32, 128, 128, 3), device="cuda")
+    ms = time_launches(timer, lambda i: fk.resize_crop_tiles(img4k, (1280, 720), rects4, out4, (1 / 255.,) * 3), steps, warmup)
+    record("C4_resize_crop_32x128x128", ms, 32 * 128 * 128, 32 * 383 * 383 * 3 + 32 * 128 * 128 * 12)
+
+    # C5: four chains over one 8192x8192 uchar4 image in one launch
+    big = rnd_u8(8192, 8192, 4)
+    gray = torch.empty((8192, 8192), dtype=torch.uint8, device="cuda")
+    small = torch.empty((512, 512, 4), device="cuda")
+    crop = torch.empty((1024, 1024, 4), dtype=torch.uint8, device="cuda")
+    bgr = torch.empty((8192, 8192, 3), device="cuda")
+    n5 = max(3, steps // 4)
+    ms = time_launches(timer, lambda i: fk.divergent4_u8c4(big, gray, small, 1 / 255., (3584, 3584, 1024, 1024), 2, crop, 0.5, bgr),
+                       n5, max(1, warmup // 4))
+    record("C5_divergent4_8192x8192", ms, 8192 * 8192 * 2 + 512 * 512 + 1024 * 1024, 1426063360,
+           "1,157,627,904 B if chains a and d share the source through cache")
+    return res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the depth sweep and the other configs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (planes/row bands would shard with no "
+                 "exchange); run with --gpus 1")
+
+    import numpy as np
+    import torch
+    import fusedkernellibrary_amd as fk
+    from oracle import binding
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    rt, _ = fk.load()
+    timer = StreamTimer(rt, torch.cuda.current_stream().cuda_stream)
+
+    src_host = binding.oracle().unit_floats(2, (H, W, 3))
+    sets = 3
+    srcs = [torch.from_numpy(src_host).cuda() for _ in range(sets)]
+    dsts = [torch.empty((H, W, 3), device="cuda") for _ in range(sets)]
+    torch.cuda.synchronize()
+
+    def step(i):
+        fk.muladd_chain_f32c3(srcs[i % sets], dsts[i % sets], DEPTH, MUL_V, ADD_V)
+
+    # timed region: exactly `steps` launches, device-synchronised on both sides
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    timer.start()
+    for i in range(args.steps):
+        step(i)
+    kernel_ms = timer.stop_ms() / args.steps
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # the result of the last timed step is the real chain (spot check against the oracle on a few rows)
+    want = binding.oracle().muladd_chain_f32c3(src_host[:4], DEPTH, MUL_V, ADD_V)
+    got = dsts[(args.steps - 1) % sets][:4].cpu().numpy()
+    assert got.tobytes() == want.tobytes(), "benchmark output differs from the oracle"
+
+    alg_bytes = 2 * W * H * 12
+    out = {
+        "metric": "fused pipeline Gpixel/s + achieved HBM GB/s (% of peak) on 1 MI355X",
+        "value": W * H / wall_ms / 1e6, "unit": "Gpixel/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"C2 vertical fusion: {W}x{H} float3, PerThreadRead -> {DEPTH} alternating Mul/Add -> "
+                               "PerThreadWrite, one fused launch per step, 3 rotating buffer sets"},
+        "roofline": {"bound": "hbm", "achieved": alg_bytes / (kernel_ms * 1e-3) / 1e9, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": alg_bytes / (kernel_ms * 1e-3) / HBM_PEAK, "traffic": None,
+                     "kernel": "transform_kernel<PointwiseJob<float3 -> float3, depth 16>>", "alg_bytes_per_launch": alg_bytes,
+                     "kernel_ms": kernel_ms},
+    }
+
+    if not args.no_sweep:
+        sweep = {}
+        k = max(10, args.steps // 4)
+        for depth in fk.CHAIN_DEPTHS:
+            fused = time_launches(timer, lambda i: fk.muladd_chain_f32c3(srcs[i % sets], dsts[i % sets], depth, MUL_V, ADD_V), k, 3)
+
+            def unfused(i):
+                a, b = srcs[i % sets], dsts[i % sets]
+                fk.single_op_f32c3(a, b, 0, MUL_V)
+                for j in range(1, depth):
+                    b2 = dsts[(i + 1) % sets] if j % 2 else dsts[i % sets]
+                    fk.single_op_f32c3(b, b2, j % 2, ADD_V if j % 2 else MUL_V)
+                    b = b2
+            unf = time_launches(timer, unfused, max(3, k // 4), 1)
+            sweep[str(depth)] = {"fused_ms": fused, "unfused_ms": unf, "fused_gb_s": alg_bytes / fused / 1e6,
+                                 "fused_frac_hbm_peak": alg_bytes / (fused * 1e-3) / HBM_PEAK, "speedup_vs_unfused": unf / fused}
+        out["depth_sweep"] = sweep
+        del srcs, dsts
+        torch.cuda.empty_cache()
+        out["other_configs"] = other_configs(fk, timer, args.steps, args.warmup)
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(src_host)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

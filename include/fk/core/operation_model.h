@@ -304,22 +304,39 @@ using get_type_t = typename detail::TupleElement<INDEX, Tuple>::type;
 
 // ---- FusedOperation -----------------------------------------------------------------------------------------
 namespace detail {
-// Runs the compute operations of a tuple in order on `input`.
+// Runs the compute operations of a tuple in order on `input`.  The tuple is only ever walked by reference, so a
+// long chain stays in the registers (or kernel-argument scalars) it arrived in.
 template <typename Input, typename Op, typename... Rest_>
 FK_HD_CNST auto tuple_compute(const Input& input, const OperationTuple<Op, Rest_...>& t) {
     static_assert(isComputeType<Op>, "Only compute operations can follow the first operation of a fused chain.");
+    using Tuple = OperationTuple<Op, Rest_...>;
     if constexpr (sizeof...(Rest_) == 0) {
         if constexpr (isUnaryType<Op>) {
             return Op::exec(input);
         } else {
             return Op::exec(input, t.instance);
         }
-    } else {
+    } else if constexpr (Tuple::HAS_NEXT) {
         if constexpr (isUnaryType<Op>) {
-            return tuple_compute(Op::exec(input), tuple_tail(t));
+            return tuple_compute(Op::exec(input), t.next);
         } else {
-            return tuple_compute(Op::exec(input, t.instance), tuple_tail(t));
+            return tuple_compute(Op::exec(input, t.instance), t.next);
         }
+    } else { // the rest is Unary only and holds no data
+        if constexpr (isUnaryType<Op>) {
+            return tuple_compute(Op::exec(input), OperationTuple<Rest_...>{});
+        } else {
+            return tuple_compute(Op::exec(input, t.instance), OperationTuple<Rest_...>{});
+        }
+    }
+}
+// Same, starting after the first element of the tuple (the read of a fused read chain).
+template <typename Input, typename Op, typename... Rest_>
+FK_HD_CNST auto tuple_compute_after_first(const Input& input, const OperationTuple<Op, Rest_...>& t) {
+    if constexpr (OperationTuple<Op, Rest_...>::HAS_NEXT) {
+        return tuple_compute(input, t.next);
+    } else {
+        return tuple_compute(input, OperationTuple<Rest_...>{});
     }
 }
 template <typename... Ops>
@@ -367,7 +384,7 @@ public:
         if constexpr (sizeof...(ComputeOps) == 0) {
             return FirstOp::exec(thread, params.instance);
         } else {
-            return detail::tuple_compute(FirstOp::exec(thread, params.instance), detail::tuple_tail(params));
+            return detail::tuple_compute_after_first(FirstOp::exec(thread, params.instance), params);
         }
     }
     FK_HD_STATIC OutputType exec(const Point& thread, const OperationDataType& opData) { return exec(thread, opData.params); }

@@ -163,7 +163,19 @@ struct PointwiseJob {
     using Src = typename View::Source;
     using OutPixel = typename Out::Pixel;
     static constexpr int K = pixels_per_thread<Src, OutPixel, Out::IS_SPLIT>();
-    static constexpr int LDS_BYTES = 0;
+    static constexpr int IN_BYTES = K * static_cast<int>(sizeof(Src));
+    static constexpr int OUT_BYTES = Out::IS_SPLIT ? K * static_cast<int>(sizeof(VBase<OutPixel>)) : K * static_cast<int>(sizeof(OutPixel));
+    // A thread's K pixels span more than one 16-byte transaction when pixels are 12 bytes wide (48 bytes per thread).
+    // Lanes reading 48-byte runs touch every cache line three times; instead the block moves its contiguous
+    // 256*K-pixel span with fully coalesced 16-byte accesses and redistributes pixels to threads through LDS.
+    static constexpr bool STAGE_IN = IN_BYTES > 16 && IN_BYTES % 16 == 0;
+    static constexpr bool STAGE_OUT = !Out::IS_SPLIT && OUT_BYTES > 16 && OUT_BYTES % 16 == 0;
+    static constexpr int STAGE_BYTES = (STAGE_IN && STAGE_OUT) ? (IN_BYTES > OUT_BYTES ? IN_BYTES : OUT_BYTES)
+                                       : STAGE_IN              ? IN_BYTES
+                                       : STAGE_OUT             ? OUT_BYTES
+                                                               : 0;
+    static constexpr int LDS_BYTES = BLOCK_THREADS * STAGE_BYTES;
+    static constexpr bool READ_IN_PLACE = N > 1 || sizeof(Prog) > 512; // run-time plane index, or a very long chain
     struct Plane {
         Prog prog;
         unsigned flags;
@@ -173,22 +185,70 @@ struct PointwiseJob {
     unsigned tx_shift; // log2 of the thread columns of a block; the other threads cover further rows
     unsigned grid_x, grid_y;
 
-    __device__ static inline void run(const PointwiseJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char*) {
-        const Plane& pl = job.plane[bz];
+    __device__ static inline void run(const PointwiseJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char* lds) {
+        const Plane& pl = job.plane[N == 1 ? 0u : bz];
         const View& v = pl.prog.view;
         const int tid = dev::thread_in_block();
         const int cols = 1 << job.tx_shift;
         const int x0 = (static_cast<int>(bx) * cols + (tid & (cols - 1))) * K;
         const int y = static_cast<int>(by) * (BLOCK_THREADS >> job.tx_shift) + (tid >> job.tx_shift);
+
+        if constexpr (STAGE_IN || STAGE_OUT) {
+            // block-uniform: the whole block lies on one row and its 256*K pixels are all inside the plane
+            const bool whole = (pl.flags & FLAG_VECTOR_IO) != 0u && job.tx_shift == 8u && y < v.h &&
+                               (static_cast<int>(bx) + 1) * BLOCK_THREADS * K <= v.w;
+            if (whole) {
+                const int bx0 = static_cast<int>(bx) * BLOCK_THREADS * K; // first pixel of the block
+                dev::u32x4* const stage = reinterpret_cast<dev::u32x4*>(lds);
+                Src in[K];
+                if constexpr (STAGE_IN) {
+                    const dev::u32x4* const g = reinterpret_cast<const dev::u32x4*>(
+                        reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy + y) * v.pitch +
+                        static_cast<size_t>(v.ox + bx0) * sizeof(Src));
+#pragma unroll
+                    for (int j = 0; j < IN_BYTES / 16; ++j) stage[j * BLOCK_THREADS + tid] = g[j * BLOCK_THREADS + tid];
+                    dev::block_sync();
+                    dev::u32x4 mine[IN_BYTES / 16];
+#pragma unroll
+                    for (int j = 0; j < IN_BYTES / 16; ++j) mine[j] = stage[tid * (IN_BYTES / 16) + j];
+                    __builtin_memcpy(in, mine, IN_BYTES);
+                } else {
+                    const char* const srow = reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy + y) * v.pitch +
+                                             static_cast<size_t>(v.ox) * sizeof(Src);
+                    unsigned int w[IN_BYTES / 4];
+                    dev::load_words<IN_BYTES>(srow + static_cast<size_t>(x0) * sizeof(Src), w);
+                    __builtin_memcpy(in, w, IN_BYTES);
+                }
+                OutPixel o[K];
+#pragma unroll
+                for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
+                if constexpr (STAGE_OUT) {
+                    if constexpr (STAGE_IN) dev::block_sync(); // every thread has taken its input out of the buffer
+                    dev::u32x4 mine[OUT_BYTES / 16];
+                    __builtin_memcpy(mine, o, OUT_BYTES);
+#pragma unroll
+                    for (int j = 0; j < OUT_BYTES / 16; ++j) stage[tid * (OUT_BYTES / 16) + j] = mine[j];
+                    dev::block_sync();
+                    dev::u32x4* const g = reinterpret_cast<dev::u32x4*>(
+                        reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
+                        static_cast<size_t>(y) * job.out.pitch + static_cast<size_t>(bx0) * sizeof(OutPixel));
+#pragma unroll
+                    for (int j = 0; j < OUT_BYTES / 16; ++j) g[j * BLOCK_THREADS + tid] = stage[j * BLOCK_THREADS + tid];
+                } else {
+                    dev::store_group<K>(job.out, x0, y, static_cast<int>(bz), o);
+                }
+                return;
+            }
+        }
+
         if (y >= v.h || x0 >= v.w) return; // also ends blocks that lie outside a smaller plane of a ragged batch
         const char* const srow = reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy + y) * v.pitch +
                                  static_cast<size_t>(v.ox) * sizeof(Src);
         if ((pl.flags & FLAG_VECTOR_IO) != 0u && x0 + K <= v.w) {
-            constexpr int NB = K * static_cast<int>(sizeof(Src));
-            unsigned int w[NB / 4];
-            dev::load_words<NB>(srow + static_cast<size_t>(x0) * sizeof(Src), w);
+            unsigned int w[IN_BYTES / 4];
+            dev::load_words<IN_BYTES>(srow + static_cast<size_t>(x0) * sizeof(Src), w);
             Src in[K];
-            __builtin_memcpy(in, w, NB);
+            __builtin_memcpy(in, w, IN_BYTES);
             OutPixel o[K];
 #pragma unroll
             for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
@@ -236,12 +296,13 @@ struct ResizeJob {
     using Pixel = typename View::Pixel;
     using OutPixel = typename Out::Pixel;
     static constexpr int LDS_BYTES = (RESIZE_LDS_DWORDS + 2) * 4;
+    static constexpr bool READ_IN_PLACE = N > 1;
     Prog plane[N];
     Out out;
     unsigned grid_x, grid_y;
 
     __device__ static inline void run(const ResizeJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char* lds_raw) {
-        const Prog& prog = job.plane[bz];
+        const Prog& prog = job.plane[N == 1 ? 0u : bz];
         const View& v = prog.view;
         const PlainView<Src>& s = v.src;
         const int tx0 = static_cast<int>(bx) * RESIZE_TILE_W;
@@ -358,6 +419,7 @@ struct ResizeJob {
 template <typename Sender, typename Receiver>
 struct GenericJob {
     static constexpr int LDS_BYTES = 0;
+    static constexpr bool READ_IN_PLACE = isBatchOperation<typename Sender::Operation>;
     Sender sender;
     Receiver receiver;
     ActiveThreads active;
@@ -377,10 +439,23 @@ struct GenericJob {
 // ---- entry points ------------------------------------------------------------------------------------------------
 extern __shared__ unsigned char fk_dynamic_lds[];
 
+// The job is the kernel's only argument, so it starts the kernel-argument segment.  It is read in place there
+// (uniform, scalar loads) rather than through the by-value parameter: a plane picked with a run-time index would
+// otherwise force a private copy of the whole job into scratch memory.
+template <typename Job>
+__device__ inline const Job& job_in_kernarg() {
+    return *(const Job*)__builtin_amdgcn_kernarg_segment_ptr();
+}
+
 template <typename Job>
 __global__ __attribute__((amdgpu_flat_work_group_size(BLOCK_THREADS, BLOCK_THREADS))) void transform_kernel(const Job job) {
-    Job::run(job, __builtin_amdgcn_workgroup_id_x(), __builtin_amdgcn_workgroup_id_y(), __builtin_amdgcn_workgroup_id_z(),
-             fk_dynamic_lds);
+    if constexpr (Job::READ_IN_PLACE) {
+        Job::run(job_in_kernarg<Job>(), __builtin_amdgcn_workgroup_id_x(), __builtin_amdgcn_workgroup_id_y(),
+                 __builtin_amdgcn_workgroup_id_z(), fk_dynamic_lds);
+    } else {
+        Job::run(job, __builtin_amdgcn_workgroup_id_x(), __builtin_amdgcn_workgroup_id_y(), __builtin_amdgcn_workgroup_id_z(),
+                 fk_dynamic_lds);
+    }
 }
 // Same, with the job read from device memory: for jobs too large for the kernel-argument segment.
 template <typename Job>
