@@ -52,8 +52,20 @@ def build_capi(extra_defines=(), name="libfk_capi.so"):
     return out
 
 
+def build_cpp_tests():
+    """The C++ programs under tests/cpp: the host-side API conformance check and the README example as user code."""
+    tests = os.path.join(ROOT, "tests", "cpp")
+    outs = []
+    for name in ("conformance", "readme_dropin"):
+        out = os.path.join(tests, name)
+        _run([hipcc(), "-x", "hip", os.path.join(tests, name + ".cpp"), "-I" + INCLUDE, *DEVICE_FLAGS, "-L" + HERE, "-lfk_hip_rt",
+              "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/../../fusedkernellibrary_amd", "-o", out])
+        outs.append(out)
+    return outs
+
+
 def build_all():
-    return [build_runtime(), build_capi()]
+    return [build_runtime(), build_capi()] + build_cpp_tests()
 
 
 if __name__ == "__main__":

@@ -66,9 +66,9 @@ template <typename IOp> using GetOutputType_t = typename IOp::Operation::OutputT
 
 namespace detail {
 template <typename T, typename = void>
-struct HasExec : std::false_type {};
+struct IsBuilderOnly : std::false_type {};
 template <typename T>
-struct HasExec<T, std::void_t<decltype(&T::exec)>> : std::true_type {};
+struct IsBuilderOnly<T, std::enable_if_t<T::BUILDER_ONLY>> : std::true_type {};
 template <typename T, typename = void>
 struct HasBatch : std::false_type {};
 template <typename T>
@@ -79,7 +79,7 @@ template <typename T>
 struct IsFused<T, std::enable_if_t<T::IS_FUSED_OP>> : std::true_type {};
 } // namespace detail
 // An operation is complete when it can execute; Crop<void>, Resize<..., void> are builders waiting for their back read.
-template <typename T> constexpr bool isCompleteOperation = detail::HasExec<T>::value;
+template <typename T> constexpr bool isCompleteOperation = isOperation<T> && !detail::IsBuilderOnly<T>::value;
 template <typename Op> constexpr bool isBatchOperation = detail::HasBatch<Op>::value;
 template <typename Op> using is_fused_operation = detail::IsFused<Op>;
 

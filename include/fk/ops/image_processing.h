@@ -139,6 +139,7 @@ private:
 
 public:
     FK_STATIC_STRUCT(Crop, SelfType)
+    static constexpr bool BUILDER_ONLY = true; // executes only once completed with its back read
     using ReadDataType = NullType;
     using OutputType = NullType;
     using ParamsType = Rect;
@@ -380,6 +381,7 @@ private:
 
 public:
     FK_STATIC_STRUCT(Resize, SelfType)
+    static constexpr bool BUILDER_ONLY = true;
     using ReadDataType = NullType;
     using OutputType = std::conditional_t<std::is_void_v<T>, NullType, T>;
     using ParamsType = IncompleteResizeReadParams<AR, T>;
@@ -422,6 +424,7 @@ private:
 public:
     FK_STATIC_STRUCT(Resize, SelfType)
     using InstanceType = ReadBackType;
+    static constexpr bool BUILDER_ONLY = true;
 
     template <typename BF, AspectRatio AR_ = AR, std::enable_if_t<AR_ == AspectRatio::IGNORE_AR && isAnyReadType<BF>, int> = 0>
     static inline constexpr auto build(const BF& backIOp, const Size& dstSize) {

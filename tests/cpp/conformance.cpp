@@ -1,0 +1,179 @@
+// Host-side conformance of the fk:: operator API: type identities, sizes and values that user code written against
+// the Fused Kernel Library relies on (the reference pins the same facts in its compile-time tests: tests/algorithm/
+// test_crop.h:28-45, tests/operation/test_instantiable_operations.h:46-226, tests/operation/test_fused_operation.h:
+// 49-116, tests/operation/test_operation_types.h:56-182, tests/data/test_rect.h:19-39, tests/data/test_ptr_nd.h:44-108).
+// Needs no GPU: everything here is compile-time or host memory.  Exit code 0 = pass.
+#include <fused_kernel/fused_kernel.h>
+
+#include <cstdio>
+#include <cstring>
+
+using namespace fk;
+
+#define EXPECT(cond)                                                                                                   \
+    do {                                                                                                               \
+        if (!(cond)) {                                                                                                 \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);                                              \
+            ++failures;                                                                                                \
+        }                                                                                                              \
+    } while (0)
+
+// ---- vector types and operators -------------------------------------------------------------------------------
+static_assert(sizeof(uchar3) == 3 && sizeof(uchar4) == 4 && alignof(uchar4) == 4 && sizeof(float3) == 12 && alignof(float3) == 4);
+static_assert(sizeof(float2) == 8 && alignof(float2) == 8 && sizeof(float4) == 16 && alignof(float4) == 16 && alignof(short4) == 8);
+static_assert(cn<uchar3> == 3 && cn<float> == 1 && cn<const uchar3> == 1);
+static_assert(std::is_same_v<VBase<float4>, float> && std::is_same_v<VectorType_t<float, 3>, float3> && std::is_same_v<VectorType_t<uchar, 1>, uchar>);
+static_assert(std::is_same_v<decltype(uchar3{} * uchar3{}), int3>, "integer promotion per channel");
+static_assert(std::is_same_v<decltype(uchar3{} * 2.f), float3> && std::is_same_v<decltype(uchar4{} * 2), int4>);
+static_assert(std::is_same_v<decltype(float3{} == float3{}), bool3>);
+static_assert((make_<float3>(1, 2, 3) + make_set<float3>(1.f)).z == 4.f);
+static_assert((uchar3{ 200, 100, 7 } * uchar3{ 2, 2, 2 }).x == 400, "no wrap-around: channels promote to int");
+
+// ---- kinds ---------------------------------------------------------------------------------------------------
+using ReadU3 = PerThreadRead<ND::_2D, uchar3>;
+static_assert(isReadType<ReadU3> && isReadType<Read<ReadU3>> && !isReadBackType<ReadU3> && isAnyReadType<Crop<Read<ReadU3>>>);
+static_assert(isReadBackType<Crop<Read<ReadU3>>> && isReadBackType<Crop<>> && !isCompleteOperation<Crop<>> && isCompleteOperation<Crop<Read<ReadU3>>>);
+static_assert(isBinaryType<Mul<float3>> && isUnaryType<Cast<uchar3, float3>> && isWriteType<TensorWrite<float3>> && isComputeType<Mul<float>>);
+static_assert(allUnaryTypes<Cast<int, float>, Cast<float, int>> && notAllUnaryTypes<Cast<int, float>, Mul<float>>);
+static_assert(noneWriteType<ReadU3, Mul<float3>> && !noneAnyWriteType<ReadU3, TensorWrite<float3>>);
+static_assert(std::is_same_v<Instantiable<Mul<float>>, Binary<Mul<float>>> && std::is_same_v<Instantiable<ReadU3>, Read<ReadU3>>);
+
+// ---- data ----------------------------------------------------------------------------------------------------
+static_assert(Rect(16, 32, 32, 64).x == 16 && Rect(16, 32, 32, 64).y == 32 && Rect(16, 32, 32, 64).width == 32 && Rect(16, 32, 32, 64).height == 64);
+static_assert(Rect().x == 0 && Rect().height == 0 && Point().z == 0 && Size(3, 4).height == 4);
+static_assert(Rect_<float, double>(1.f, 2.f, 3., 4.).width == 3.);
+
+// ---- chains --------------------------------------------------------------------------------------------------
+constexpr RawPtr<ND::_2D, uchar3> kInput{ nullptr, PtrDims<ND::_2D>(128, 64, 128 * 3) };
+constexpr auto kRead = ReadU3::build(kInput);
+static_assert(kRead.getActiveThreads() == ActiveThreads(128, 64, 1));
+
+constexpr auto kCrop = kRead.then(Crop<>::build(Rect(5, 6, 30, 20)));
+static_assert(std::is_same_v<std::decay_t<decltype(kCrop)>, ReadBack<Crop<Read<ReadU3>>>> && kCrop.getActiveThreads() == ActiveThreads(30, 20, 1));
+static_assert(std::is_same_v<std::decay_t<decltype(Crop<Read<ReadU3>>::build(kRead, Rect(1, 1, 2, 2)))>, ReadBack<Crop<Read<ReadU3>>>>);
+
+constexpr std::array<Rect, 2> kTwoCrops{ Rect(0, 0, 34, 25), Rect(10, 10, 70, 15) };
+constexpr auto kBatchResize = kRead.then(Crop<>::build(kTwoCrops)).then(Resize<InterpolationType::INTER_LINEAR>::build(Size(100, 100)));
+static_assert(kBatchResize.getActiveThreads() == ActiveThreads(100, 100, 2));
+static_assert(std::decay_t<decltype(kBatchResize)>::Operation::BATCH == 2 && !isBatchOperation<std::decay_t<decltype(kCrop)>::Operation>);
+
+// five operations fuse flat, never nested
+constexpr auto kFive = kRead.then(Cast<uchar3, float3>::build())
+                           .then(Mul<float3>::build(make_set<float3>(2.f)))
+                           .then(Cast<float3, int3>::build())
+                           .then(Cast<int3, float3>::build());
+using FiveOp = std::decay_t<decltype(kFive)>::Operation;
+static_assert(std::is_same_v<FiveOp, FusedOperation<ReadU3, Cast<uchar3, float3>, Mul<float3>, Cast<float3, int3>, Cast<int3, float3>>>);
+static_assert(FiveOp::ParamsType::size == 5 && kFive.params.next.next.instance.params.y == 2.f, "Binary parameters reachable through next");
+static_assert(sizeof(OperationTuple<Cast<int, float>, Cast<float, int>>) == 1, "Unary operations occupy no storage");
+static_assert(FusedOperation<Cast<float, int>, Cast<int, float>>::exec(5.5f) == 5.f, "an all-Unary chain runs in constant expressions");
+static_assert(std::is_same_v<std::decay_t<decltype(Add<int>::build(4).then(Add<int>::build(4)).then(Add<int>::build(3)))>::Operation::InstanceType, BinaryType>);
+static_assert(std::decay_t<decltype(Add<int>::build(4).then(Add<int>::build(4)).then(Add<int>::build(3)))>::Operation::exec(
+                  0, Add<int>::build(4).then(Add<int>::build(4)).then(Add<int>::build(3))) == 11);
+
+// operations before a ReadBack fold into its back read; a compute operation after it gives a plain fused read
+constexpr auto kCastResize = kRead.then(Cast<uchar3, float3>::build()).then(Resize<InterpolationType::INTER_LINEAR>::build(Size(16, 16)));
+static_assert(isReadBackType<std::decay_t<decltype(kCastResize)>>);
+static_assert(std::is_same_v<std::decay_t<decltype(kCastResize.backIOp)>::Operation, FusedOperation<ReadU3, Cast<uchar3, float3>>>);
+static_assert(isReadType<std::decay_t<decltype(kCastResize.then(Mul<float3>::build(make_set<float3>(1.f))))>>);
+
+// the README chain
+constexpr std::array<Rect, 5> kReadmeCrops{ Rect(0, 0, 34, 25), Rect(10, 10, 70, 15), Rect(20, 20, 60, 59), Rect(30, 30, 20, 23), Rect(40, 40, 12, 11) };
+constexpr RawPtr<ND::_2D, uchar3> k4K{ nullptr, PtrDims<ND::_2D>(3840, 2160, 3840 * 3) };
+constexpr auto kReadme = ReadU3::build(k4K)
+                             .then(Crop<>::build(kReadmeCrops))
+                             .then(Resize<InterpolationType::INTER_LINEAR, AspectRatio::PRESERVE_AR>::build(Size(60, 60), float3{ 0.f, 0.f, 0.f }))
+                             .then(Mul<float3>::build(make_set<float3>(1.4f)))
+                             .then(Sub<float3>::build(make_set<float3>(0.5f)))
+                             .then(Div<float3>::build(make_set<float3>(255.f)))
+                             .then(ColorConversion<ColorConversionCodes::COLOR_RGB2BGR, float3, float3>::build());
+using ReadmeResize = Resize<InterpolationType::INTER_LINEAR, AspectRatio::PRESERVE_AR, ReadBack<Crop<Read<ReadU3>>>>;
+static_assert(std::is_same_v<std::decay_t<decltype(kReadme)>,
+                             Read<BatchRead<5, PlanePolicy::PROCESS_ALL,
+                                            FusedOperation<ReadmeResize, Mul<float3>, Sub<float3>, Div<float3>, VectorReorder<float3, 2, 1, 0>>>>>);
+static_assert(sizeof(kReadme) == 696, "same parameter block size as the reference's README chain");
+static_assert(kReadme.getActiveThreads() == ActiveThreads(60, 60, 5));
+static_assert(kReadme.params.opData[3].params.instance.params.x1 == 4 && kReadme.params.opData[3].params.instance.params.x2 == 55 &&
+              kReadme.params.opData[0].params.instance.params.y1 == 8 && kReadme.params.opData[0].params.instance.params.y2 == 51);
+
+// conditional batches keep usedPlanes / default_value through then()
+constexpr std::array<Size, 3> kSizes{ Size(8, 8), Size(8, 8), Size(8, 8) };
+constexpr std::array<RawPtr<ND::_2D, uchar3>, 3> kThree{ kInput, kInput, kInput };
+constexpr auto kCond = ReadU3::build(2, uchar3{ 1, 2, 3 }, kThree);
+static_assert(std::decay_t<decltype(kCond)>::Operation::PP == PlanePolicy::CONDITIONAL_WITH_DEFAULT && kCond.params.usedPlanes == 2 && kCond.params.default_value.z == 3);
+constexpr auto kCondResized = kCond.then(Resize<InterpolationType::INTER_LINEAR>::build(Size(8, 8)));
+static_assert(kCondResized.params.usedPlanes == 2 && kCondResized.params.default_value.y == 2.f, "default cast to the new output type");
+constexpr std::array<Read<ReadU3>, 3> kThreeReads{ kRead, kRead, kRead };
+static_assert(std::decay_t<decltype(Resize<InterpolationType::INTER_LINEAR>::build(kThreeReads, kSizes))>::Operation::BATCH == 3);
+
+// DPP tags
+static_assert(TransformDPP<>::PAR_ARCH == ParArch::GPU_AMD && defaultParArch == ParArch::GPU_AMD && Stream::parArch() == ParArch::GPU_AMD);
+static_assert(exec::pixels_per_thread<float3, float3, false>() == 4 && exec::pixels_per_thread<uchar4, uchar, false>() == 4 &&
+              exec::pixels_per_thread<uchar4, float3, false>() == 4 && exec::pixels_per_thread<uchar, uchar, false>() == 16);
+
+int main() {
+    int failures = 0;
+    // owning host buffers: refcount through copies, crop views share ownership, at() addresses by pitch
+    {
+        Ptr2D<uchar3> img(64, 32, 0, MemType::Host);
+        EXPECT(img.getRefCount() == 1 && img.dims().pitch == 64 * 3 && img.sizeInBytes() == 64u * 32u * 3u);
+        {
+            Ptr2D<uchar3> copy = img;
+            EXPECT(img.getRefCount() == 2);
+            auto view = copy.crop2D(Point(4, 2), PtrDims<ND::_2D>(8, 8));
+            EXPECT(img.getRefCount() == 3 && view.dims().pitch == img.dims().pitch);
+            img.at(4, 2) = uchar3{ 9, 8, 7 };
+            EXPECT(view.at(0, 0).x == 9 && view.at(0, 0).z == 7);
+        }
+        EXPECT(img.getRefCount() == 1);
+        Tensor<float3> t(6, 5, 4, 1, MemType::Host);
+        EXPECT(t.dims().pitch == 6 * sizeof(float3) && t.dims().plane_pitch == 6 * 5 * sizeof(float3) && t.getNumElements() == 120);
+        t.at(1, 2, 3) = float3{ 1.f, 2.f, 3.f };
+        auto plane = t.getPlane(3);
+        EXPECT(plane.at(1, 2).y == 2.f && t.getRefCount() == 2);
+    }
+    // misuse throws, as the reference's Ptr does
+    {
+        bool threw = false;
+        try {
+            uchar3 pixel{};
+            Ptr2D<uchar3> bad(&pixel, 1, 1, 3, MemType::DeviceAndPinned);
+        } catch (const std::runtime_error&) {
+            threw = true;
+        }
+        EXPECT(threw);
+        threw = false;
+        try {
+            Ptr2D<uchar3> host(4, 4, 0, MemType::Host), other(4, 4, 0, MemType::Host);
+            host.uploadTo(other); // destination is not device memory
+        } catch (const std::runtime_error&) {
+            threw = true;
+        }
+        EXPECT(threw);
+        threw = false;
+        try {
+            Ptr2D<uchar3> twice(4, 4, 0, MemType::Host);
+            twice.Alloc(Size(4, 4), 0, MemType::Host);
+        } catch (const std::runtime_error&) {
+            threw = true;
+        }
+        EXPECT(threw);
+    }
+    // host evaluation of a chain element by element (the operations are plain host+device functions)
+    {
+        Ptr2D<uchar3> img(16, 16, 0, MemType::Host);
+        for (uint y = 0; y < 16; ++y)
+            for (uint x = 0; x < 16; ++x) img.at(x, y) = uchar3{ static_cast<uchar>(x), static_cast<uchar>(y), 5 };
+        const auto chain = PerThreadRead<ND::_2D, uchar3>::build(img.ptrPinned())
+                               .then(Crop<>::build(Rect(2, 3, 8, 8)))
+                               .then(Resize<InterpolationType::INTER_LINEAR>::build(Size(8, 8)))
+                               .then(ColorConversion<ColorConversionCodes::COLOR_RGB2BGR, float3, float3>::build());
+        const float3 v = std::decay_t<decltype(chain)>::Operation::exec(Point(1, 2), chain);
+        EXPECT(v.x == 5.f && v.y == 5.f && v.z == 3.f); // identity resize of the crop, channels reversed
+        const auto view = exec::ViewOf<std::decay_t<decltype(PerThreadRead<ND::_2D, uchar3>::build(img.ptrPinned()).then(Crop<>::build(Rect(2, 3, 8, 8))))>>::make(
+            PerThreadRead<ND::_2D, uchar3>::build(img.ptrPinned()).then(Crop<>::build(Rect(2, 3, 8, 8))));
+        EXPECT(view.ox == 2 && view.oy == 3 && view.w == 8 && view.h == 8 && view.img_w == 16);
+    }
+    if (failures == 0) std::printf("conformance ok\n");
+    return failures == 0 ? 0 : 1;
+}

@@ -1,0 +1,34 @@
+"""The C++ side as a user sees it: programs under tests/cpp compiled against include/ by the build step."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from conftest import same_bits
+from oracle import binding as B
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def test_host_api_conformance():
+    exe = os.path.join(HERE, "cpp", "conformance")
+    assert os.path.exists(exe), "tests/cpp/conformance is not built (python -m fusedkernellibrary_amd.build)"
+    proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
+    assert proc.returncode == 0, proc.stdout
+    assert "conformance ok" in proc.stdout
+
+
+@pytest.mark.gpu
+def test_readme_example_as_user_code(oracle, tmp_path):
+    exe = os.path.join(HERE, "cpp", "readme_dropin")
+    assert os.path.exists(exe), "tests/cpp/readme_dropin is not built"
+    src = oracle.bytes(1, (2160, 3840, 3))
+    fin, fout = tmp_path / "in.bin", tmp_path / "out.bin"
+    src.tofile(fin)
+    proc = subprocess.run([exe, str(fin), str(fout)], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert proc.returncode == 0, proc.stdout
+    got = np.fromfile(fout, np.float32).reshape(5, 60, 60, 3)
+    rects = [(0, 0, 34, 25), (10, 10, 70, 15), (20, 20, 60, 59), (30, 30, 20, 23), (40, 40, 12, 11)]
+    want = oracle.crop_resize_muls_bgr_tensor(src, rects, (60, 60), B.PRESERVE_AR, (0, 0, 0), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)
+    assert same_bits(got, want)

@@ -1,0 +1,155 @@
+"""GPU parity on the awkward shapes: ragged and tiny inputs, odd widths, padded pitches, unaligned views, every tail
+path of the vectorised kernels, large batches (kernel-argument blocks beyond 4 KiB) and argument errors."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import same_bits
+from oracle import binding as B
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def padded(a, extra):
+    """Copy `a` (h, w, c) into a device buffer whose rows are `extra` pixels longer: pitch != width * pixel size."""
+    h, w, c = a.shape
+    buf = torch.zeros((h, w + extra, c), dtype=torch.from_numpy(a).dtype, device="cuda")
+    buf[:, :w] = torch.from_numpy(a).cuda()
+    return buf[:, :w]
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (1, 3), (3, 1), (7, 5), (1, 1023), (1, 1024), (1, 1025), (2, 4097), (33, 257), (64, 256)])
+def test_pointwise_every_tail(fk, oracle, shape):
+    h, w = shape
+    src = oracle.unit_floats(2, (h, w, 3))
+    out = torch.full((h, w, 3), float("nan"), device="cuda")
+    fk.muladd_chain_f32c3(dev(src), out, 4, 1.0001, 1e-4)
+    torch.cuda.synchronize()
+    assert same_bits(out.cpu().numpy(), oracle.muladd_chain_f32c3(src, 4, 1.0001, 1e-4))
+
+
+@pytest.mark.parametrize("extra", [1, 4, 13])
+def test_pointwise_padded_and_unaligned_rows(fk, oracle, extra):
+    src = oracle.unit_floats(2, (37, 1100, 3))
+    want = oracle.muladd_chain_f32c3(src, 2, 1.0001, 1e-4)
+    s = padded(src, extra)
+    full = torch.full((37, 1100 + extra, 3), float("nan"), device="cuda")
+    out = full[:, :1100]
+    fk.muladd_chain_f32c3(s, out, 2, 1.0001, 1e-4)
+    torch.cuda.synchronize()
+    assert same_bits(out.cpu().numpy(), want)
+    assert torch.isnan(full[:, 1100:]).all()  # nothing written past the row end
+    # a view that starts 1 pixel (12 bytes) into the row: base no longer 16-byte aligned
+    s2, o2 = s[:, 1:], out[:, 1:]
+    fk.muladd_chain_f32c3(s2, o2, 2, 1.0001, 1e-4)
+    torch.cuda.synchronize()
+    assert same_bits(o2.cpu().numpy(), want[:, 1:])
+
+
+def test_uchar4_chains_odd_sizes_and_pitch(fk, oracle):
+    src = oracle.bytes(5, (61, 203, 4))
+    s = padded(src, 3)
+    gray_full = torch.zeros((61, 203 + 5), dtype=torch.uint8, device="cuda")
+    fk.rgba2gray_u8c4(s, gray_full[:, :203])
+    bgr = torch.full((61, 203, 3), float("nan"), device="cuda")
+    fk.rgba2bgr_sub_u8c4_f32c3(s, bgr, 0.5)
+    rect = (17, 9, 150, 40)
+    crop = torch.zeros((40, 150, 4), dtype=torch.uint8, device="cuda")
+    fk.crop_mul_saturate_u8c4(s, rect, crop, 3)
+    small = torch.full((7, 11, 4), float("nan"), device="cuda")
+    fk.resize_mul_u8c4_f32c4(s, small, 1 / 255.)
+    up = torch.full((200, 333, 4), float("nan"), device="cuda")
+    fk.resize_mul_u8c4_f32c4(s, up, 1.0)
+    torch.cuda.synchronize()
+    assert same_bits(gray_full[:, :203].cpu().numpy(), oracle.rgba2gray_u8c4(src)) and (gray_full[:, 203:] == 0).all()
+    assert same_bits(bgr.cpu().numpy(), oracle.rgba2bgr_sub_u8c4_f32c3(src, 0.5))
+    assert same_bits(crop.cpu().numpy(), oracle.crop_mul_saturate_u8c4(src, rect, 3))
+    assert same_bits(small.cpu().numpy(), oracle.resize_mul_u8c4_f32c4(src, (11, 7), 1 / 255.))
+    assert same_bits(up.cpu().numpy(), oracle.resize_mul_u8c4_f32c4(src, (333, 200), 1.0))
+
+
+@pytest.mark.parametrize("aspect", [B.PRESERVE_AR, B.IGNORE_AR, B.PRESERVE_AR_RN_EVEN, B.PRESERVE_AR_LEFT])
+@pytest.mark.parametrize("n", [1, 2, 3, 8])
+def test_readme_chain_tiny_and_extreme_crops(fk, oracle, aspect, n):
+    h, w = 97, 131
+    src = oracle.bytes(40 + n, (h, w, 3))
+    pool = [(0, 0, 1, 1), (130, 96, 1, 1), (0, 0, 131, 97), (5, 7, 2, 90), (3, 3, 120, 2), (64, 32, 33, 17), (1, 1, 129, 95), (100, 0, 31, 97)]
+    rects = pool[:n]
+    for dst in ((1, 1), (37, 53), (256, 9)):
+        args = (aspect, (0.25, -1.0, 3.0), (1.4, 0.7, 2.0), (0.5, 0.1, -0.3), (255., 3., 0.5))
+        want = oracle.crop_resize_muls_bgr_tensor(src, rects, dst, *args)
+        out = torch.full((n, dst[1], dst[0], 3), float("nan"), device="cuda")
+        fk.crop_resize_muls_bgr_tensor(padded(src, 1), rects, out, *args)
+        torch.cuda.synchronize()
+        assert same_bits(out.cpu().numpy(), want), (dst, aspect, n)
+
+
+def test_large_batches_exceed_four_kib_of_kernel_arguments(fk, oracle):
+    for n in (32, 50):
+        src = oracle.bytes(60, (200, 300, 3))
+        rects = [((7 * i) % 200, (5 * i) % 120, 16 + (11 * i) % 80, 8 + (13 * i) % 70) for i in range(n)]
+        args = (B.PRESERVE_AR, (0, 0, 0), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)
+        want = oracle.crop_resize_muls_bgr_tensor(src, rects, (40, 24), *args)
+        out = torch.full((n, 24, 40, 3), float("nan"), device="cuda")
+        fk.crop_resize_muls_bgr_tensor(dev(src), rects, out, *args)
+        torch.cuda.synchronize()
+        assert same_bits(out.cpu().numpy(), want), n
+
+
+def test_split_and_tiles_small_batches(fk, oracle):
+    for n in (1, 2, 3, 8):
+        srcs = [oracle.bytes(70 + i, (90, 160, 3)) for i in range(n)]
+        rects = [(3 * i, 2 * i, 20 + 15 * i, 11 + 9 * i) for i in range(n)]
+        args = ((255.,) * 3, (.485, .456, .406), (.229, .224, .225))
+        out = torch.full((n, 3, 30, 50), float("nan"), device="cuda")
+        fk.batch_crop_resize_norm_split([dev(s) for s in srcs], rects, out, *args)
+        torch.cuda.synchronize()
+        assert same_bits(out.cpu().numpy(), oracle.batch_crop_resize_norm_split(srcs, rects, (50, 30), *args)), n
+        src = oracle.gradient_noise_u8c3(4, 200, 120)
+        tiles = [(4 * i, 3 * i, 9, 7) for i in range(n)]
+        o2 = torch.full((n, 7, 9, 3), float("nan"), device="cuda")
+        fk.resize_crop_tiles(dev(src), (50, 40), tiles, o2, (1 / 255.,) * 3)
+        torch.cuda.synchronize()
+        assert same_bits(o2.cpu().numpy(), oracle.resize_crop_tiles(src, (50, 40), tiles, (9, 7), (1 / 255.,) * 3)), n
+
+
+def test_upscale_of_crops_with_odd_byte_offsets(fk, oracle):
+    # crops starting at every byte phase of a uchar3 row, tight and padded pitches: the LDS staging aligns rows itself
+    src = oracle.bytes(80, (70, 101, 3))
+    for extra in (0, 1, 2, 3):
+        s = padded(src, extra) if extra else dev(src)
+        rects = [(x, 3 + x, 37, 29) for x in (0, 1, 2, 3, 4)]
+        out = torch.full((5, 120, 150, 3), float("nan"), device="cuda")
+        args = (B.IGNORE_AR, (0, 0, 0), (1.0,) * 3, (0.0,) * 3, (1.0,) * 3)
+        fk.crop_resize_muls_bgr_tensor(s, rects, out, *args)
+        torch.cuda.synchronize()
+        assert same_bits(out.cpu().numpy(), oracle.crop_resize_muls_bgr_tensor(src, rects, (150, 120), *args)), extra
+
+
+def test_crop_at_the_last_row_and_column_of_the_buffer(fk, oracle):
+    # the source window ends exactly at the end of the allocation: staging must not read past it
+    src = oracle.bytes(81, (33, 47, 3))
+    rects = [(20, 10, 27, 23), (46, 32, 1, 1)]
+    out = torch.full((2, 64, 64, 3), float("nan"), device="cuda")
+    args = (B.PRESERVE_AR, (1.0, 2.0, 3.0), (1.0,) * 3, (0.0,) * 3, (1.0,) * 3)
+    fk.crop_resize_muls_bgr_tensor(dev(src), rects, out, *args)
+    torch.cuda.synchronize()
+    assert same_bits(out.cpu().numpy(), oracle.crop_resize_muls_bgr_tensor(src, rects, (64, 64), *args))
+
+
+def test_argument_errors(fk, oracle):
+    src = dev(oracle.bytes(1, (20, 30, 3)))
+    out = torch.zeros((4, 8, 8, 3), device="cuda")
+    with pytest.raises(fk.FkError, match="unsupported"):
+        fk.crop_resize_muls_bgr_tensor(src, [(0, 0, 4, 4)] * 4, out, 0, (0,) * 3, (1,) * 3, (0,) * 3, (1,) * 3)
+    out = torch.zeros((1, 8, 8, 3), device="cuda")
+    with pytest.raises(fk.FkError, match="outside"):
+        fk.crop_resize_muls_bgr_tensor(src, [(25, 0, 10, 4)], out, 0, (0,) * 3, (1,) * 3, (0,) * 3, (1,) * 3)
+    with pytest.raises(fk.FkError, match="unsupported"):
+        f = torch.zeros((4, 4, 3), device="cuda")
+        fk.muladd_chain_f32c3(f, f.clone(), 3, 1.0, 1.0)
+    torch.cuda.synchronize()
