@@ -142,6 +142,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the depth sweep and the other configs")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run plain device copies of the same 99.5 MB image (torch copy kernel) before the timed "
+                         "region, so that a counter run has a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (planes/row bands would shard with no "
@@ -165,6 +168,11 @@ def main():
 
     def step(i):
         fk.muladd_chain_f32c3(srcs[i % sets], dsts[i % sets], DEPTH, MUL_V, ADD_V)
+
+    if args.copy_calibration:
+        for i in range(10):
+            dsts[i % sets].copy_(srcs[i % sets])
+        torch.cuda.synchronize()
 
     # timed region: exactly `steps` launches, device-synchronised on both sides
     for i in range(args.warmup):

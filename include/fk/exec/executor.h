@@ -43,6 +43,7 @@ inline constexpr auto buildOperationSequence(const First& first, const Rest&... 
 namespace exec {
 
 inline unsigned ceil_div(unsigned a, unsigned b) { return (a + b - 1u) / b; }
+constexpr size_t STREAM_STORE_MIN_BYTES = 32u << 20; // about the aggregate L2 of the eight XCDs
 inline bool aligned_to(const void* p, size_t a) { return reinterpret_cast<size_t>(p) % a == 0; }
 
 // ---- job construction ----------------------------------------------------------------------------------------
@@ -120,7 +121,9 @@ struct JobOf {
                     const char* const ofirst = reinterpret_cast<const char*>(out.data) + i * out.z_stride;
                     vec = vec && aligned_to(ofirst, out_chunk) && (v.h == 1 || out.pitch % out_chunk == 0);
                     if constexpr (Out::IS_SPLIT) vec = vec && out.chan_stride % out_chunk == 0;
-                    job.plane[i].flags = vec ? FLAG_VECTOR_IO : 0u;
+                    // outputs larger than the caches are written with streaming stores
+                    const bool stream = static_cast<size_t>(v.w) * v.h * N * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
+                    job.plane[i].flags = (vec ? FLAG_VECTOR_IO : 0u) | (vec && stream ? FLAG_STREAM_STORES : 0u);
                     max_w = v.w > max_w ? v.w : max_w;
                     max_h = v.h > max_h ? v.h : max_h;
                 }

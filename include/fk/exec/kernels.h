@@ -67,7 +67,18 @@ __device__ inline void load_words(const void* p, unsigned int* w) {
         for (int i = 0; i < NBYTES / 4; ++i) w[i] = static_cast<const unsigned int*>(p)[i];
     }
 }
-template <int NBYTES>
+// STREAM: non-temporal stores.  Only for accesses where a wave writes whole cache lines (consecutive lanes,
+// consecutive 16/8/4-byte pieces): they then leave the caches alone and measurably raise the write bandwidth;
+// on partial lines they are a pessimisation.
+template <bool STREAM, typename V>
+__device__ inline void store_piece(V* p, const V& v) {
+    if constexpr (STREAM) {
+        __builtin_nontemporal_store(v, p);
+    } else {
+        *p = v;
+    }
+}
+template <int NBYTES, bool STREAM = false>
 __device__ inline void store_words(void* p, const unsigned int* w) {
     constexpr int C = chunk_bytes(NBYTES);
     static_assert(NBYTES % 4 == 0 && C >= 4, "vector I/O moves whole dwords");
@@ -76,18 +87,18 @@ __device__ inline void store_words(void* p, const unsigned int* w) {
         for (int i = 0; i < NBYTES / 16; ++i) {
             u32x4 v;
             v.x = w[4 * i]; v.y = w[4 * i + 1]; v.z = w[4 * i + 2]; v.w = w[4 * i + 3];
-            static_cast<u32x4*>(p)[i] = v;
+            store_piece<STREAM>(static_cast<u32x4*>(p) + i, v);
         }
     } else if constexpr (C == 8) {
 #pragma unroll
         for (int i = 0; i < NBYTES / 8; ++i) {
             u32x2 v;
             v.x = w[2 * i]; v.y = w[2 * i + 1];
-            static_cast<u32x2*>(p)[i] = v;
+            store_piece<STREAM>(static_cast<u32x2*>(p) + i, v);
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < NBYTES / 4; ++i) static_cast<unsigned int*>(p)[i] = w[i];
+        for (int i = 0; i < NBYTES / 4; ++i) store_piece<STREAM>(static_cast<unsigned int*>(p) + i, w[i]);
     }
 }
 
@@ -116,15 +127,16 @@ __device__ inline void store_one(const SplitOut<O>& out, int x, int y, int z, co
 }
 
 // K consecutive pixels starting at x0 (caller guarantees the alignment that chunk_bytes asks for)
-template <int K, typename O>
+template <int K, bool STREAM = false, typename O>
 __device__ inline void store_group(const PackedOut<O>& out, int x0, int y, int z, const O* v) {
     constexpr int NB = K * static_cast<int>(sizeof(O));
     unsigned int w[NB / 4];
     __builtin_memcpy(w, v, NB);
     char* const row = reinterpret_cast<char*>(out.data) + static_cast<size_t>(z) * out.z_stride + static_cast<size_t>(y) * out.pitch;
-    store_words<NB>(row + static_cast<size_t>(x0) * sizeof(O), w);
+    // a thread's K pixels are one transaction only when they fill exactly one piece
+    store_words<NB, STREAM && NB == chunk_bytes(NB)>(row + static_cast<size_t>(x0) * sizeof(O), w);
 }
-template <int K, typename O>
+template <int K, bool STREAM = false, typename O>
 __device__ inline void store_group(const SplitOut<O>& out, int x0, int y, int z, const O* v) {
     using B = VBase<O>;
     constexpr int NB = K * static_cast<int>(sizeof(B));
@@ -136,7 +148,7 @@ __device__ inline void store_group(const SplitOut<O>& out, int x0, int y, int z,
         for (int k = 0; k < K; ++k) ch[k] = vectorAt(c, v[k]);
         unsigned int w[NB / 4];
         __builtin_memcpy(w, ch, NB);
-        store_words<NB>(row + c * out.chan_stride + static_cast<size_t>(x0) * sizeof(B), w);
+        store_words<NB, STREAM && NB == chunk_bytes(NB)>(row + c * out.chan_stride + static_cast<size_t>(x0) * sizeof(B), w);
     }
 }
 } // namespace dev
@@ -155,7 +167,7 @@ constexpr int pixels_per_thread() {
 }
 
 // ---- pointwise ---------------------------------------------------------------------------------------------------
-enum : unsigned { FLAG_VECTOR_IO = 1u };
+enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u };
 
 template <typename Prog, size_t N, typename Out>
 struct PointwiseJob {
@@ -232,10 +244,16 @@ struct PointwiseJob {
                     dev::u32x4* const g = reinterpret_cast<dev::u32x4*>(
                         reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
                         static_cast<size_t>(y) * job.out.pitch + static_cast<size_t>(bx0) * sizeof(OutPixel));
+                    if ((pl.flags & FLAG_STREAM_STORES) != 0u) {
 #pragma unroll
-                    for (int j = 0; j < OUT_BYTES / 16; ++j) g[j * BLOCK_THREADS + tid] = stage[j * BLOCK_THREADS + tid];
+                        for (int j = 0; j < OUT_BYTES / 16; ++j) dev::store_piece<true>(g + j * BLOCK_THREADS + tid, stage[j * BLOCK_THREADS + tid]);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < OUT_BYTES / 16; ++j) g[j * BLOCK_THREADS + tid] = stage[j * BLOCK_THREADS + tid];
+                    }
                 } else {
-                    dev::store_group<K>(job.out, x0, y, static_cast<int>(bz), o);
+                    if ((pl.flags & FLAG_STREAM_STORES) != 0u) dev::store_group<K, true>(job.out, x0, y, static_cast<int>(bz), o);
+                    else dev::store_group<K>(job.out, x0, y, static_cast<int>(bz), o);
                 }
                 return;
             }
@@ -252,7 +270,8 @@ struct PointwiseJob {
             OutPixel o[K];
 #pragma unroll
             for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
-            dev::store_group<K>(job.out, x0, y, static_cast<int>(bz), o);
+            if ((pl.flags & FLAG_STREAM_STORES) != 0u) dev::store_group<K, true>(job.out, x0, y, static_cast<int>(bz), o);
+            else dev::store_group<K>(job.out, x0, y, static_cast<int>(bz), o);
         } else {
             const int xe = x0 + K < v.w ? x0 + K : v.w;
             for (int x = x0; x < xe; ++x) {
