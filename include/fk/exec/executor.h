@@ -94,6 +94,17 @@ struct JobOf {
                 job.out = out;
                 job.grid_x = ceil_div(static_cast<unsigned>(max_w), RESIZE_TILE_W);
                 job.grid_y = ceil_div(static_cast<unsigned>(max_h), RESIZE_TILE_H);
+                // vector stores need 16-byte aligned rows in every plane (tiles start at multiples of 64 pixels)
+                constexpr size_t out_elem = Out::IS_SPLIT ? sizeof(VBase<typename Out::Pixel>) : sizeof(typename Out::Pixel);
+                bool vec = aligned_to(out.data, 16) && out.pitch % 16 == 0 && out.z_stride % 16 == 0 && (RESIZE_TILE_W * out_elem) % 16 == 0;
+                if constexpr (Out::IS_SPLIT) vec = vec && out.chan_stride % 16 == 0;
+                const bool stream = static_cast<size_t>(max_w) * max_h * N * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
+                job.flags = (vec ? FLAG_VECTOR_IO : 0u) | (vec && stream ? FLAG_STREAM_STORES : 0u);
+                for (size_t i = 0; i < N; ++i) {
+                    if (decltype(job)::worth_staging(job.plane[i].view.fx, job.plane[i].view.fy)) job.flags |= FLAG_SOURCE_TILE;
+                }
+                // small outputs gain nothing from leaving through LDS, and the LDS they would ask for lowers occupancy
+                if (vec && static_cast<size_t>(max_w) * max_h * N * sizeof(typename Out::Pixel) >= (1u << 20)) job.flags |= FLAG_STAGE_OUT;
                 return job;
             } else {
                 using Job = PointwiseJob<Prog, N, Out>;
@@ -174,7 +185,7 @@ inline void launch_args(const void* by_value, const void* indirect, const Args& 
 template <typename Job>
 inline void launch_job(const Job& job, unsigned planes, fkrt_stream stream) {
     launch_args(reinterpret_cast<const void*>(&transform_kernel<Job>), reinterpret_cast<const void*>(&transform_kernel_indirect<Job>),
-                job, job.grid_x, job.grid_y, planes, Job::LDS_BYTES, stream);
+                job, job.grid_x, job.grid_y, planes, job.lds_bytes(), stream);
 }
 
 // (read, compute..., write) as (sender, receiver)
@@ -290,8 +301,7 @@ private:
         pack.job = Plan::make(seq.sender, seq.receiver);
         pack.blocks = pack.job.grid_x * pack.job.grid_y * Plan::planes(seq.sender);
         total += pack.blocks;
-        using Job = std::decay_t<decltype(pack.job)>;
-        lds = lds > static_cast<size_t>(Job::LDS_BYTES) ? lds : static_cast<size_t>(Job::LDS_BYTES);
+        lds = lds > pack.job.lds_bytes() ? lds : pack.job.lds_bytes();
         fill(pack.rest, total, lds, rest...);
     }
 };

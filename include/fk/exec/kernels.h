@@ -3,10 +3,11 @@
 // Every launch runs blocks of 256 threads (four wave64).  A "job" is one fused chain over all its planes:
 //   PointwiseJob  element-wise chains over a PlainView: each thread owns K consecutive pixels of a row so that both the
 //                 source and the destination bytes of a thread are whole 16-byte (or 8/4-byte) transactions;
-//   ResizeJob     bilinear resize (with optional inner/outer crop and aspect-ratio border): a block owns a 32x8 output
-//                 tile, stages the source bounding box of the tile in LDS with coalesced dword loads and takes the
-//                 2x2 taps from LDS; tiles whose bounding box does not fit (strong down-scaling, no tap reuse) read
-//                 their taps straight from memory;
+//   ResizeJob     bilinear resize (with optional inner/outer crop and aspect-ratio border): a block owns a 64x16 output
+//                 tile, four pixels per thread; it stages the source bounding box of the tile in LDS, one dword-aligned
+//                 slot per source pixel, and takes the 2x2 taps from there; tiles that gain nothing from it (strong
+//                 down-scaling, no tap reuse) read their taps straight from memory; packed outputs leave through LDS
+//                 as whole 16-byte pieces;
 //   GenericJob    one thread per output element through Operation::exec, for any chain the views cannot describe.
 // blockIdx.z selects the plane of a batch; blocks that start outside their plane's own extent return at once.
 // What one thread computes per element is the reference's TransformDPP::exec -> read -> compute... -> write
@@ -34,8 +35,8 @@ namespace dev {
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
-__device__ inline int thread_in_block() { return static_cast<int>(__builtin_amdgcn_workitem_id_x()); }
-__device__ inline void block_sync() {
+__device__ __attribute__((always_inline)) inline int thread_in_block() { return static_cast<int>(__builtin_amdgcn_workitem_id_x()); }
+__device__ __attribute__((always_inline)) inline void block_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
@@ -47,7 +48,7 @@ constexpr int chunk_bytes(int nbytes) { return gcd(nbytes, 16); }
 
 // NBYTES (a multiple of 4) from `p`, which is aligned to chunk_bytes(NBYTES)
 template <int NBYTES>
-__device__ inline void load_words(const void* p, unsigned int* w) {
+__device__ __attribute__((always_inline)) inline void load_words(const void* p, unsigned int* w) {
     constexpr int C = chunk_bytes(NBYTES);
     static_assert(NBYTES % 4 == 0 && C >= 4, "vector I/O moves whole dwords");
     if constexpr (C == 16) {
@@ -71,7 +72,7 @@ __device__ inline void load_words(const void* p, unsigned int* w) {
 // consecutive 16/8/4-byte pieces): they then leave the caches alone and measurably raise the write bandwidth;
 // on partial lines they are a pessimisation.
 template <bool STREAM, typename V>
-__device__ inline void store_piece(V* p, const V& v) {
+__device__ __attribute__((always_inline)) inline void store_piece(V* p, const V& v) {
     if constexpr (STREAM) {
         __builtin_nontemporal_store(v, p);
     } else {
@@ -79,7 +80,7 @@ __device__ inline void store_piece(V* p, const V& v) {
     }
 }
 template <int NBYTES, bool STREAM = false>
-__device__ inline void store_words(void* p, const unsigned int* w) {
+__device__ __attribute__((always_inline)) inline void store_words(void* p, const unsigned int* w) {
     constexpr int C = chunk_bytes(NBYTES);
     static_assert(NBYTES % 4 == 0 && C >= 4, "vector I/O moves whole dwords");
     if constexpr (C == 16) {
@@ -103,7 +104,7 @@ __device__ inline void store_words(void* p, const unsigned int* w) {
 }
 
 template <typename Tail, typename V>
-__device__ inline auto apply_tail(const Tail& tail, const V& v) {
+__device__ __attribute__((always_inline)) inline auto apply_tail(const Tail& tail, const V& v) {
     if constexpr (std::is_same_v<Tail, NoTail>) {
         return v;
     } else {
@@ -112,12 +113,12 @@ __device__ inline auto apply_tail(const Tail& tail, const V& v) {
 }
 
 template <typename O>
-__device__ inline void store_one(const PackedOut<O>& out, int x, int y, int z, const O& v) {
+__device__ __attribute__((always_inline)) inline void store_one(const PackedOut<O>& out, int x, int y, int z, const O& v) {
     char* const row = reinterpret_cast<char*>(out.data) + static_cast<size_t>(z) * out.z_stride + static_cast<size_t>(y) * out.pitch;
     reinterpret_cast<O*>(row)[x] = v;
 }
 template <typename O>
-__device__ inline void store_one(const SplitOut<O>& out, int x, int y, int z, const O& v) {
+__device__ __attribute__((always_inline)) inline void store_one(const SplitOut<O>& out, int x, int y, int z, const O& v) {
     using B = VBase<O>;
     char* const row = reinterpret_cast<char*>(out.data) + static_cast<size_t>(z) * out.z_stride + static_cast<size_t>(y) * out.pitch;
     reinterpret_cast<B*>(row)[x] = v.x;
@@ -128,7 +129,7 @@ __device__ inline void store_one(const SplitOut<O>& out, int x, int y, int z, co
 
 // K consecutive pixels starting at x0 (caller guarantees the alignment that chunk_bytes asks for)
 template <int K, bool STREAM = false, typename O>
-__device__ inline void store_group(const PackedOut<O>& out, int x0, int y, int z, const O* v) {
+__device__ __attribute__((always_inline)) inline void store_group(const PackedOut<O>& out, int x0, int y, int z, const O* v) {
     constexpr int NB = K * static_cast<int>(sizeof(O));
     unsigned int w[NB / 4];
     __builtin_memcpy(w, v, NB);
@@ -137,7 +138,7 @@ __device__ inline void store_group(const PackedOut<O>& out, int x0, int y, int z
     store_words<NB, STREAM && NB == chunk_bytes(NB)>(row + static_cast<size_t>(x0) * sizeof(O), w);
 }
 template <int K, bool STREAM = false, typename O>
-__device__ inline void store_group(const SplitOut<O>& out, int x0, int y, int z, const O* v) {
+__device__ __attribute__((always_inline)) inline void store_group(const SplitOut<O>& out, int x0, int y, int z, const O* v) {
     using B = VBase<O>;
     constexpr int NB = K * static_cast<int>(sizeof(B));
     char* const row = reinterpret_cast<char*>(out.data) + static_cast<size_t>(z) * out.z_stride + static_cast<size_t>(y) * out.pitch;
@@ -167,7 +168,7 @@ constexpr int pixels_per_thread() {
 }
 
 // ---- pointwise ---------------------------------------------------------------------------------------------------
-enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u };
+enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_STAGE_OUT = 8u };
 
 template <typename Prog, size_t N, typename Out>
 struct PointwiseJob {
@@ -196,8 +197,9 @@ struct PointwiseJob {
     Out out;
     unsigned tx_shift; // log2 of the thread columns of a block; the other threads cover further rows
     unsigned grid_x, grid_y;
+    size_t lds_bytes() const { return LDS_BYTES; }
 
-    __device__ static inline void run(const PointwiseJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char* lds) {
+    __device__ __attribute__((always_inline)) static inline void run(const PointwiseJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char* lds) {
         const Plane& pl = job.plane[N == 1 ? 0u : bz];
         const View& v = pl.prog.view;
         const int tid = dev::thread_in_block();
@@ -283,28 +285,62 @@ struct PointwiseJob {
 };
 
 // ---- resize ------------------------------------------------------------------------------------------------------
-constexpr int RESIZE_TILE_W = 32;
-constexpr int RESIZE_TILE_H = 8;
-constexpr int RESIZE_LDS_DWORDS = 4096;
+// A block owns a 64x16 output tile of one plane; a thread computes four consecutive pixels of one row, so everything
+// that depends only on the row (or only on the column) is computed once and shared.
+constexpr int RESIZE_TILE_W = 64;
+constexpr int RESIZE_TILE_H = 16;
+constexpr int RESIZE_PX = 4;                // pixels per thread, along x
+constexpr int RESIZE_LDS_DWORDS = 6144;     // source tile capacity (24 KiB)
 
 namespace dev {
-// sizeof(T) bytes at byte offset `off` of a dword array in LDS
+// LDS slot of one source pixel: whole dwords, so a tap is one aligned LDS read whatever the pixel's byte size
 template <typename T>
-__device__ inline T lds_pixel(const unsigned int* tile, unsigned off) {
-    constexpr int ND = (static_cast<int>(sizeof(T)) + 3) / 4;
-    const unsigned int* const p = tile + (off >> 2);
-    const unsigned sh = off & 3u;
-    unsigned int w[ND];
-    if constexpr (sizeof(T) % 4 == 0 && alignof(T) % 4 == 0) {
-#pragma unroll
-        for (int i = 0; i < ND; ++i) w[i] = p[i]; // such pixels only ever sit at dword offsets
-    } else {
-#pragma unroll
-        for (int i = 0; i < ND; ++i) w[i] = __builtin_amdgcn_alignbyte(p[i + 1], p[i], sh);
-    }
+constexpr int slot_dwords() { return (static_cast<int>(sizeof(T)) + 3) / 4; }
+
+template <typename T>
+struct PixelSlot {
+    unsigned int w[slot_dwords<T>()];
+};
+template <typename T>
+__device__ __attribute__((always_inline)) inline T slot_to_pixel(const PixelSlot<T>& s) {
     T out;
-    __builtin_memcpy(&out, w, sizeof(T));
+    __builtin_memcpy(&out, s.w, sizeof(T));
     return out;
+}
+// One pixel from memory at any byte alignment, as whole dwords.  `row` points at byte 0 of the window row, `off` is the
+// pixel's byte offset in it; [valid_lo, valid_hi) are the byte offsets of that row that belong to the parent image, so
+// dwords that would reach past them are assembled from single bytes.
+template <typename T>
+__device__ __attribute__((always_inline)) inline PixelSlot<T> load_pixel_slot(const char* row, int off, int valid_lo, int valid_hi) {
+    constexpr int ND = slot_dwords<T>();
+    PixelSlot<T> s;
+    if constexpr (alignof(T) % 4 == 0) {
+        const unsigned int* const p = reinterpret_cast<const unsigned int*>(row + off);
+#pragma unroll
+        for (int i = 0; i < ND; ++i) s.w[i] = p[i];
+    } else {
+        const unsigned mis = (static_cast<unsigned>(reinterpret_cast<size_t>(row)) + static_cast<unsigned>(off)) & 3u;
+        const int first = off - static_cast<int>(mis); // aligned dword that holds the pixel's first byte
+        const bool spills = mis + sizeof(T) > 4u * ND;  // the pixel reaches into one more dword
+        if (first >= valid_lo && first + 4 * (ND + (spills ? 1 : 0)) <= valid_hi) {
+            const unsigned int* const p = reinterpret_cast<const unsigned int*>(row + first);
+            unsigned int lo = p[0];
+#pragma unroll
+            for (int i = 0; i < ND; ++i) {
+                const unsigned int hi = (i + 1 < ND || spills) ? p[i + 1] : 0u;
+                s.w[i] = __builtin_amdgcn_alignbyte(hi, lo, mis);
+                lo = hi;
+            }
+        } else { // at the edge of the parent image: byte by byte
+#pragma unroll
+            for (int i = 0; i < ND; ++i) s.w[i] = 0u;
+#pragma unroll
+            for (int b = 0; b < static_cast<int>(sizeof(T)); ++b) {
+                s.w[b / 4] |= static_cast<unsigned int>(static_cast<unsigned char>(row[off + b])) << (8 * (b % 4));
+            }
+        }
+    }
+    return s;
 }
 } // namespace dev
 
@@ -314,13 +350,84 @@ struct ResizeJob {
     using Src = typename View::Source;
     using Pixel = typename View::Pixel;
     using OutPixel = typename Out::Pixel;
-    static constexpr int LDS_BYTES = (RESIZE_LDS_DWORDS + 2) * 4;
+    static constexpr int SLOT = dev::slot_dwords<Src>();
+    static constexpr int OUT_ROW_BYTES = RESIZE_TILE_W * static_cast<int>(sizeof(OutPixel));
+    // packed outputs whose four pixels per thread are not one 16-byte piece go out through LDS as whole 16-byte pieces
+    static constexpr bool STAGE_OUT = !Out::IS_SPLIT && (RESIZE_PX * sizeof(OutPixel)) % 16 == 0 && RESIZE_PX * sizeof(OutPixel) > 16;
+    static constexpr int OUT_STAGE_BYTES = STAGE_OUT ? RESIZE_TILE_H * OUT_ROW_BYTES : 0;
+    static constexpr int LDS_BYTES = (RESIZE_LDS_DWORDS * 4 > OUT_STAGE_BYTES ? RESIZE_LDS_DWORDS * 4 : OUT_STAGE_BYTES) + 16;
     static constexpr bool READ_IN_PLACE = N > 1;
     Prog plane[N];
     Out out;
     unsigned grid_x, grid_y;
+    // FLAG_VECTOR_IO: output rows start 16-byte aligned; FLAG_STREAM_STORES: large output; FLAG_SOURCE_TILE: some plane's
+    // tiles are worth staging in LDS; FLAG_STAGE_OUT: packed output leaves through LDS.  The last two decide how much
+    // LDS the launch asks for (a divergent launch shares one LDS size between all its jobs).
+    unsigned flags;
+    size_t lds_bytes() const {
+        size_t n = 0;
+        if ((flags & FLAG_SOURCE_TILE) != 0u) n = RESIZE_LDS_DWORDS * 4;
+        if (STAGE_OUT && (flags & FLAG_STAGE_OUT) != 0u && static_cast<size_t>(OUT_STAGE_BYTES) > n) n = OUT_STAGE_BYTES;
+        return n == 0 ? 0 : n + 16;
+    }
+    // whether a tile of a plane with these factors can be staged (same rule as the kernel applies per tile)
+    static bool worth_staging(float fx, float fy) {
+        const int cols = static_cast<int>((RESIZE_TILE_W - 1) * fx) + 3, rows = static_cast<int>((RESIZE_TILE_H - 1) * fy) + 3;
+        return rows * (cols | 1) * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * RESIZE_TILE_W * RESIZE_TILE_H + 256;
+    }
 
-    __device__ static inline void run(const ResizeJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char* lds_raw) {
+    // Four consecutive pixels of row y, taps from the staged tile (STAGED) or straight from memory.
+    template <bool STAGED>
+    __device__ __attribute__((always_inline)) static inline void pixels(const Prog& prog, const unsigned int* tile, const char* window,
+                                                                       int sx_lo, int sy_lo, int stride, int x_first, int y, OutPixel* o) {
+        const View& v = prog.view;
+        const PlainView<Src>& s = v.src;
+        const int ry = y + v.off_y;
+        bool row_inside = y < v.h;
+        if constexpr (View::HAS_ROI) row_inside = row_inside && ry >= v.y1 && ry <= v.y2;
+        const float src_y = (ry - v.y1) * v.fy;
+#pragma unroll
+        for (int k = 0; k < RESIZE_PX; ++k) {
+            const int x = x_first + k;
+            const int rx = x + v.off_x;
+            bool inside = row_inside && x < v.w;
+            if constexpr (View::HAS_ROI) inside = inside && rx >= v.x1 && rx <= v.x2;
+            Pixel value = v.background;
+            if (inside) {
+                const float src_x = (rx - v.x1) * v.fx;
+                const fk::detail::BilinearTaps t = fk::detail::bilinear_taps(src_x, src_y, Size(s.w, s.h));
+                Src a, b, c, d;
+                if constexpr (STAGED) {
+                    // the tile holds columns sx_lo.. and rows sy_lo.., edge copies included: no clamping here
+                    const unsigned int* const p0 = tile + ((t.y1 - sy_lo) * stride + (t.x1 - sx_lo)) * SLOT;
+                    const unsigned int* const p1 = p0 + stride * SLOT;
+                    dev::PixelSlot<Src> sa, sb, sc, sd;
+#pragma unroll
+                    for (int i = 0; i < SLOT; ++i) {
+                        sa.w[i] = p0[i];
+                        sb.w[i] = p0[SLOT + i];
+                        sc.w[i] = p1[i];
+                        sd.w[i] = p1[SLOT + i];
+                    }
+                    a = dev::slot_to_pixel<Src>(sa);
+                    b = dev::slot_to_pixel<Src>(sb);
+                    c = dev::slot_to_pixel<Src>(sc);
+                    d = dev::slot_to_pixel<Src>(sd);
+                } else {
+                    const char* const r0 = window + static_cast<size_t>(t.y1) * s.pitch;
+                    const char* const r1 = window + static_cast<size_t>(t.y2r) * s.pitch;
+                    a = reinterpret_cast<const Src*>(r0)[t.x1];
+                    b = reinterpret_cast<const Src*>(r0)[t.x2r];
+                    c = reinterpret_cast<const Src*>(r1)[t.x1];
+                    d = reinterpret_cast<const Src*>(r1)[t.x2r];
+                }
+                value = fk::detail::bilinear_blend(a, b, c, d, t);
+            }
+            o[k] = dev::apply_tail(prog.tail, value);
+        }
+    }
+
+    __device__ __attribute__((always_inline)) static inline void run(const ResizeJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char* lds_raw) {
         const Prog& prog = job.plane[N == 1 ? 0u : bz];
         const View& v = prog.view;
         const PlainView<Src>& s = v.src;
@@ -328,8 +435,8 @@ struct ResizeJob {
         const int ty0 = static_cast<int>(by) * RESIZE_TILE_H;
         if (tx0 >= v.w || ty0 >= v.h) return; // block outside this plane's own extent
         const int tid = dev::thread_in_block();
-        const int x = tx0 + (tid & (RESIZE_TILE_W - 1));
-        const int y = ty0 + (tid / RESIZE_TILE_W);
+        const int x_first = tx0 + (tid & (RESIZE_TILE_W / RESIZE_PX - 1)) * RESIZE_PX;
+        const int y = ty0 + tid / (RESIZE_TILE_W / RESIZE_PX);
 
         // part of the tile that resamples the source, in resize coordinates (after the outer crop offset)
         int rx_lo = tx0 + v.off_x, rx_hi = (tx0 + RESIZE_TILE_W < v.w ? tx0 + RESIZE_TILE_W : v.w) - 1 + v.off_x;
@@ -345,92 +452,88 @@ struct ResizeJob {
         unsigned int* const tile = reinterpret_cast<unsigned int*>(lds_raw);
         bool staged = false;
         int sx_lo = 0, sy_lo = 0;
-        unsigned stride_dw = 0;
-        const unsigned base_lo = static_cast<unsigned>(reinterpret_cast<size_t>(s.data));
+        int stride = 0; // slots per tile row
+        const char* const window = reinterpret_cast<const char*>(s.data) + static_cast<size_t>(s.oy) * s.pitch +
+                                   static_cast<size_t>(s.ox) * sizeof(Src); // window pixel (0, 0)
+        const int valid_lo = -s.ox * static_cast<int>(sizeof(Src));
+        const int valid_hi = (s.img_w - s.ox) * static_cast<int>(sizeof(Src));
 #ifndef FK_INTERPOLATE_Y1_FROM_X
         if (resamples) {
-            // source bounding box of the tile: taps are floor(c) and min(floor(c) + 1, limit) for c in [lo, hi] * f
+            // source bounding box of the tile: taps are floor(c) and floor(c) + 1 for c in [lo, hi] * f; the column and
+            // row past the source edge are staged as copies of the last one, which is what the clamp of the taps reads
             sx_lo = fk::detail::floor_to_int((rx_lo - v.x1) * v.fx);
             sy_lo = fk::detail::floor_to_int((ry_lo - v.y1) * v.fy);
-            int sx_hi = fk::detail::floor_to_int((rx_hi - v.x1) * v.fx) + 1;
-            int sy_hi = fk::detail::floor_to_int((ry_hi - v.y1) * v.fy) + 1;
-            sx_hi = sx_hi < s.w - 1 ? sx_hi : s.w - 1;
-            sy_hi = sy_hi < s.h - 1 ? sy_hi : s.h - 1;
-            sx_lo = sx_lo < sx_hi ? sx_lo : sx_hi;
-            sy_lo = sy_lo < sy_hi ? sy_lo : sy_hi;
-            const int rows = sy_hi - sy_lo + 1;
-            const unsigned row_bytes = static_cast<unsigned>(sx_hi - sx_lo + 1) * sizeof(Src);
-            stride_dw = ((row_bytes + 3u) >> 2) + 1u; // + up to 3 bytes of misalignment at the row start
-            stride_dw |= 1u;                          // odd stride spreads rows over the LDS banks
-            staged = static_cast<unsigned>(rows) * stride_dw <= static_cast<unsigned>(RESIZE_LDS_DWORDS);
+            const int cols = fk::detail::floor_to_int((rx_hi - v.x1) * v.fx) + 2 - sx_lo;
+            const int rows = fk::detail::floor_to_int((ry_hi - v.y1) * v.fy) + 2 - sy_lo;
+            stride = cols | 1;
+            const int tile_px = (rx_hi - rx_lo + 1) * (ry_hi - ry_lo + 1);
+            // staging pays off while a source pixel is used about once or more; strong down-scaling reads taps directly
+            staged = (job.flags & FLAG_SOURCE_TILE) != 0u && rows * stride * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * tile_px + 256;
             if (staged) {
                 const int wave = tid >> 6, lane = tid & 63;
-                const long valid_lo = -static_cast<long>(s.ox) * static_cast<long>(sizeof(Src));
-                const long valid_hi = static_cast<long>(s.img_w - s.ox) * static_cast<long>(sizeof(Src));
                 for (int r = wave; r < rows; r += BLOCK_THREADS / 64) {
-                    const size_t row_off = static_cast<size_t>(s.oy + sy_lo + r) * s.pitch + static_cast<size_t>(s.ox) * sizeof(Src);
-                    const char* const row = reinterpret_cast<const char*>(s.data) + row_off; // window x = 0 of this row
-                    const long first = static_cast<long>(sx_lo) * static_cast<long>(sizeof(Src));
-                    const unsigned mis = (base_lo + static_cast<unsigned>(row_off) + static_cast<unsigned>(first)) & 3u;
-                    const unsigned need = (mis + row_bytes + 3u) >> 2;
-                    for (unsigned c = static_cast<unsigned>(lane); c < need; c += 64u) {
-                        const long b = first - static_cast<long>(mis) + 4l * static_cast<long>(c); // byte offset in the window row
-                        unsigned int word;
-                        if (b >= valid_lo && b + 4 <= valid_hi) {
-                            word = *reinterpret_cast<const unsigned int*>(row + b);
-                        } else { // dword straddles the end of the parent image row: take only the bytes that exist
-                            word = 0u;
+                    const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
+                    const char* const row = window + static_cast<size_t>(sy) * s.pitch;
+                    for (int c = lane; c < cols; c += 64) {
+                        const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
+                        const dev::PixelSlot<Src> px = dev::load_pixel_slot<Src>(row, sx * static_cast<int>(sizeof(Src)), valid_lo, valid_hi);
 #pragma unroll
-                            for (int k = 0; k < 4; ++k) {
-                                if (b + k >= valid_lo && b + k < valid_hi) {
-                                    word |= static_cast<unsigned int>(static_cast<unsigned char>(row[b + k])) << (8 * k);
-                                }
-                            }
-                        }
-                        tile[static_cast<unsigned>(r) * stride_dw + c] = word;
+                        for (int i = 0; i < SLOT; ++i) tile[(r * stride + c) * SLOT + i] = px.w[i];
                     }
                 }
             }
         }
 #endif
         dev::block_sync();
-        if (x >= v.w || y >= v.h) return;
 
-        Pixel value;
-        const int rx = x + v.off_x, ry = y + v.off_y;
-        bool inside = true;
-        if constexpr (View::HAS_ROI) inside = rx >= v.x1 && rx <= v.x2 && ry >= v.y1 && ry <= v.y2;
-        if (inside) {
-            const float src_x = (rx - v.x1) * v.fx;
-            const float src_y = (ry - v.y1) * v.fy;
-            const fk::detail::BilinearTaps t = fk::detail::bilinear_taps(src_x, src_y, Size(s.w, s.h));
-            Src a, b, c, d;
-            if (staged) {
-                const unsigned row0 = static_cast<unsigned>(t.y1 - sy_lo), row1 = static_cast<unsigned>(t.y2r - sy_lo);
-                const unsigned first = static_cast<unsigned>(sx_lo) * static_cast<unsigned>(sizeof(Src));
-                const unsigned org = base_lo + static_cast<unsigned>(s.ox) * static_cast<unsigned>(sizeof(Src)) + first;
-                const unsigned mis0 = (org + static_cast<unsigned>(s.oy + t.y1) * s.pitch) & 3u;
-                const unsigned mis1 = (org + static_cast<unsigned>(s.oy + t.y2r) * s.pitch) & 3u;
-                const unsigned xa = static_cast<unsigned>(t.x1 - sx_lo) * static_cast<unsigned>(sizeof(Src));
-                const unsigned xb = static_cast<unsigned>(t.x2r - sx_lo) * static_cast<unsigned>(sizeof(Src));
-                a = dev::lds_pixel<Src>(tile, row0 * stride_dw * 4u + mis0 + xa);
-                b = dev::lds_pixel<Src>(tile, row0 * stride_dw * 4u + mis0 + xb);
-                c = dev::lds_pixel<Src>(tile, row1 * stride_dw * 4u + mis1 + xa);
-                d = dev::lds_pixel<Src>(tile, row1 * stride_dw * 4u + mis1 + xb);
-            } else {
-                const char* const r0 = reinterpret_cast<const char*>(s.data) + static_cast<size_t>(s.oy + t.y1) * s.pitch;
-                const char* const r1 = reinterpret_cast<const char*>(s.data) + static_cast<size_t>(s.oy + t.y2r) * s.pitch;
-                a = reinterpret_cast<const Src*>(r0)[s.ox + t.x1];
-                b = reinterpret_cast<const Src*>(r0)[s.ox + t.x2r];
-                c = reinterpret_cast<const Src*>(r1)[s.ox + t.x1];
-                d = reinterpret_cast<const Src*>(r1)[s.ox + t.x2r];
-            }
-            value = fk::detail::bilinear_blend(a, b, c, d, t);
+        // ---- this thread's four pixels; the tap source is decided once for the block ----
+        OutPixel o[RESIZE_PX];
+        if (staged) {
+            pixels<true>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
         } else {
-            value = v.background;
+            pixels<false>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
         }
-        const OutPixel o = dev::apply_tail(prog.tail, value);
-        dev::store_one(job.out, x, y, static_cast<int>(bz), o);
+
+        // ---- write ----
+        const bool whole_width = tx0 + RESIZE_TILE_W <= v.w; // block-uniform
+        if constexpr (STAGE_OUT) {
+            if (whole_width && (job.flags & FLAG_STAGE_OUT) != 0u) {
+                constexpr int PIECES_PER_ROW = OUT_ROW_BYTES / 16;
+                constexpr int MINE = RESIZE_PX * static_cast<int>(sizeof(OutPixel)) / 16;
+                dev::u32x4* const stage = reinterpret_cast<dev::u32x4*>(lds_raw);
+                dev::block_sync(); // every thread is done with the source tile
+                dev::u32x4 mine[MINE];
+                __builtin_memcpy(mine, o, sizeof(mine));
+#pragma unroll
+                for (int j = 0; j < MINE; ++j) stage[tid * MINE + j] = mine[j];
+                dev::block_sync();
+                char* const obase = reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
+                                    static_cast<size_t>(ty0) * job.out.pitch + static_cast<size_t>(tx0) * sizeof(OutPixel);
+                const int rows_here = v.h - ty0 < RESIZE_TILE_H ? v.h - ty0 : RESIZE_TILE_H;
+                const bool stream = (job.flags & FLAG_STREAM_STORES) != 0u;
+#pragma unroll
+                for (int j = 0; j < RESIZE_TILE_H * PIECES_PER_ROW / BLOCK_THREADS; ++j) {
+                    const int id = j * BLOCK_THREADS + tid;
+                    const int r = id / PIECES_PER_ROW, c = id - r * PIECES_PER_ROW;
+                    if (r < rows_here) {
+                        dev::u32x4* const g = reinterpret_cast<dev::u32x4*>(obase + static_cast<size_t>(r) * job.out.pitch) + c;
+                        if (stream) dev::store_piece<true>(g, stage[id]);
+                        else *g = stage[id];
+                    }
+                }
+                return;
+            }
+        }
+        if (y >= v.h) return;
+        if (x_first + RESIZE_PX <= v.w && (job.flags & FLAG_VECTOR_IO) != 0u && (Out::IS_SPLIT || RESIZE_PX * sizeof(OutPixel) == 16)) {
+            if ((job.flags & FLAG_STREAM_STORES) != 0u) dev::store_group<RESIZE_PX, true>(job.out, x_first, y, static_cast<int>(bz), o);
+            else dev::store_group<RESIZE_PX>(job.out, x_first, y, static_cast<int>(bz), o);
+        } else {
+#pragma unroll
+            for (int k = 0; k < RESIZE_PX; ++k) {
+                if (x_first + k < v.w) dev::store_one(job.out, x_first + k, y, static_cast<int>(bz), o[k]);
+            }
+        }
     }
 };
 
@@ -443,8 +546,9 @@ struct GenericJob {
     Receiver receiver;
     ActiveThreads active;
     unsigned grid_x, grid_y;
+    size_t lds_bytes() const { return 0; }
 
-    __device__ static inline void run(const GenericJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char*) {
+    __device__ __attribute__((always_inline)) static inline void run(const GenericJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char*) {
         const int tid = dev::thread_in_block();
         const int x = static_cast<int>(bx) * 64 + (tid & 63);
         const int y = static_cast<int>(by) * 4 + (tid >> 6);
@@ -462,7 +566,7 @@ extern __shared__ unsigned char fk_dynamic_lds[];
 // (uniform, scalar loads) rather than through the by-value parameter: a plane picked with a run-time index would
 // otherwise force a private copy of the whole job into scratch memory.
 template <typename Job>
-__device__ inline const Job& job_in_kernarg() {
+__device__ __attribute__((always_inline)) inline const Job& job_in_kernarg() {
     return *(const Job*)__builtin_amdgcn_kernarg_segment_ptr();
 }
 
@@ -489,14 +593,14 @@ template <typename... Jobs>
 struct JobPack;
 template <>
 struct JobPack<> {
-    __device__ static inline void run(const JobPack&, unsigned, unsigned char*) {}
+    __device__ __attribute__((always_inline)) static inline void run(const JobPack&, unsigned, unsigned char*) {}
 };
 template <typename Job, typename... Rest>
 struct JobPack<Job, Rest...> {
     Job job;
     unsigned blocks; // blocks of this job: grid_x * grid_y * planes
     JobPack<Rest...> rest;
-    __device__ static inline void run(const JobPack& pack, unsigned block, unsigned char* lds) {
+    __device__ __attribute__((always_inline)) static inline void run(const JobPack& pack, unsigned block, unsigned char* lds) {
         if (block < pack.blocks) {
             const unsigned bx = block % pack.job.grid_x;
             const unsigned q = block / pack.job.grid_x;
