@@ -104,6 +104,19 @@ def _check(rc):
         raise FkError(f"fk call failed ({kinds.get(rc, rc)}): {capi.fk_last_error().decode()}")
 
 
+def _call(fn, args, defer):
+    """Run the entry point now, or (defer=True) return a zero-argument callable that runs it with these already
+    marshalled arguments: for tight launch loops that should not pay the marshalling again."""
+    if defer:
+        def run():
+            rc = fn(*args)
+            if rc != 0:
+                _check(rc)
+        return run
+    _check(fn(*args))
+    return None
+
+
 def _stream(stream):
     if stream is not None:
         return C.c_void_p(stream)
@@ -131,37 +144,37 @@ def _image(t, dtype_name):
 
 # ---- chains: each mirrors one entry point of include/fk_capi.h; outputs are written into `out` ----------------------
 
-def crop_resize_muls_bgr_tensor(src, rects, out, aspect, background, mul, sub, div, stream=None):
+def crop_resize_muls_bgr_tensor(src, rects, out, aspect, background, mul, sub, div, stream=None, defer=False):
     """README pipeline. src: (H, W, 3) uint8; out: (n, dst_h, dst_w, 3) float32 contiguous."""
     _, capi = load()
     p, w, h, pitch = _image(src, "uint8")
     out = _dev(out, "float32")
     n, dh, dw, _ = out.shape
     assert n == len(rects) and out.is_contiguous()
-    _check(capi.fk_crop_resize_muls_bgr_tensor(p, w, h, pitch, _rects(rects), n, dw, dh, aspect, _f3(background), _f3(mul),
-                                               _f3(sub), _f3(div), C.c_void_p(out.data_ptr()), _stream(stream)))
-    return out
+    _deferred = _call(capi.fk_crop_resize_muls_bgr_tensor, (p, w, h, pitch, _rects(rects), n, dw, dh, aspect, _f3(background), _f3(mul),
+                                               _f3(sub), _f3(div), C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
 
 
-def muladd_chain_f32c3(src, dst, depth, mul_v, add_v, stream=None):
+def muladd_chain_f32c3(src, dst, depth, mul_v, add_v, stream=None, defer=False):
     _, capi = load()
     p, w, h, pitch = _image(src, "float32")
     q, w2, h2, pitch2 = _image(dst, "float32")
     assert (w, h) == (w2, h2)
-    _check(capi.fk_muladd_chain_f32c3(p, w, h, pitch, depth, mul_v, add_v, q, pitch2, _stream(stream)))
-    return dst
+    _deferred = _call(capi.fk_muladd_chain_f32c3, (p, w, h, pitch, depth, mul_v, add_v, q, pitch2, _stream(stream)), defer)
+    return _deferred if defer else dst
 
 
-def single_op_f32c3(src, dst, is_add, v, stream=None):
+def single_op_f32c3(src, dst, is_add, v, stream=None, defer=False):
     _, capi = load()
     p, w, h, pitch = _image(src, "float32")
     q, w2, h2, pitch2 = _image(dst, "float32")
     assert (w, h) == (w2, h2)
-    _check(capi.fk_single_op_f32c3(p, w, h, pitch, int(is_add), v, q, pitch2, _stream(stream)))
-    return dst
+    _deferred = _call(capi.fk_single_op_f32c3, (p, w, h, pitch, int(is_add), v, q, pitch2, _stream(stream)), defer)
+    return _deferred if defer else dst
 
 
-def batch_crop_resize_norm_split(srcs, rects, out, div1, sub, div2, stream=None):
+def batch_crop_resize_norm_split(srcs, rects, out, div1, sub, div2, stream=None, defer=False):
     """srcs: list of (H, W, 3) uint8 of one size/pitch; out: (n, 3, dst_h, dst_w) float32 contiguous."""
     _, capi = load()
     n = len(srcs)
@@ -171,73 +184,74 @@ def batch_crop_resize_norm_split(srcs, rects, out, div1, sub, div2, stream=None)
     ptrs = (C.c_void_p * n)(*[s.data_ptr() for s in srcs])
     out = _dev(out, "float32")
     assert out.shape[0] == n == len(rects) and out.shape[1] == 3 and out.is_contiguous()
-    _check(capi.fk_batch_crop_resize_norm_split(ptrs, w, h, pitch, _rects(rects), n, out.shape[3], out.shape[2], _f3(div1),
-                                                _f3(sub), _f3(div2), C.c_void_p(out.data_ptr()), _stream(stream)))
-    return out
+    _deferred = _call(capi.fk_batch_crop_resize_norm_split, (ptrs, w, h, pitch, _rects(rects), n, out.shape[3], out.shape[2], _f3(div1),
+                                                _f3(sub), _f3(div2), C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
 
 
-def resize_crop_tiles(src, resized, rects, out, mul, stream=None):
+def resize_crop_tiles(src, resized, rects, out, mul, stream=None, defer=False):
     """src: (H, W, 3) uint8; resized = (rs_w, rs_h); out: (n, tile_h, tile_w, 3) float32 contiguous."""
     _, capi = load()
     p, w, h, pitch = _image(src, "uint8")
     out = _dev(out, "float32")
     n, th, tw, _ = out.shape
     assert n == len(rects) and out.is_contiguous()
-    _check(capi.fk_resize_crop_tiles(p, w, h, pitch, resized[0], resized[1], _rects(rects), n, tw, th, _f3(mul),
-                                     C.c_void_p(out.data_ptr()), _stream(stream)))
-    return out
+    _deferred = _call(capi.fk_resize_crop_tiles, (p, w, h, pitch, resized[0], resized[1], _rects(rects), n, tw, th, _f3(mul),
+                                     C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
 
 
-def rgba2gray_u8c4(src, dst, stream=None):
+def rgba2gray_u8c4(src, dst, stream=None, defer=False):
     _, capi = load()
     p, w, h, pitch = _image(src, "uint8")
     d = _dev(dst, "uint8")
-    _check(capi.fk_rgba2gray_u8c4(p, w, h, pitch, C.c_void_p(d.data_ptr()), d.stride(0), _stream(stream)))
-    return dst
+    _deferred = _call(capi.fk_rgba2gray_u8c4, (p, w, h, pitch, C.c_void_p(d.data_ptr()), d.stride(0), _stream(stream)), defer)
+    return _deferred if defer else dst
 
 
-def resize_mul_u8c4_f32c4(src, dst, mul_v, stream=None):
+def resize_mul_u8c4_f32c4(src, dst, mul_v, stream=None, defer=False):
     _, capi = load()
     p, w, h, pitch = _image(src, "uint8")
     q, dw, dh, dpitch = _image(dst, "float32")
-    _check(capi.fk_resize_mul_u8c4_f32c4(p, w, h, pitch, dw, dh, mul_v, q, dpitch, _stream(stream)))
-    return dst
+    _deferred = _call(capi.fk_resize_mul_u8c4_f32c4, (p, w, h, pitch, dw, dh, mul_v, q, dpitch, _stream(stream)), defer)
+    return _deferred if defer else dst
 
 
-def crop_mul_saturate_u8c4(src, rect, dst, mul_v, stream=None):
+def crop_mul_saturate_u8c4(src, rect, dst, mul_v, stream=None, defer=False):
     _, capi = load()
     p, w, h, pitch = _image(src, "uint8")
     q, _, _, dpitch = _image(dst, "uint8")
-    _check(capi.fk_crop_mul_saturate_u8c4(p, w, h, pitch, Rect(*rect), mul_v, q, dpitch, _stream(stream)))
-    return dst
+    _deferred = _call(capi.fk_crop_mul_saturate_u8c4, (p, w, h, pitch, Rect(*rect), mul_v, q, dpitch, _stream(stream)), defer)
+    return _deferred if defer else dst
 
 
-def rgba2bgr_sub_u8c4_f32c3(src, dst, sub_v, stream=None):
+def rgba2bgr_sub_u8c4_f32c3(src, dst, sub_v, stream=None, defer=False):
     _, capi = load()
     p, w, h, pitch = _image(src, "uint8")
     q, _, _, dpitch = _image(dst, "float32")
-    _check(capi.fk_rgba2bgr_sub_u8c4_f32c3(p, w, h, pitch, sub_v, q, dpitch, _stream(stream)))
-    return dst
+    _deferred = _call(capi.fk_rgba2bgr_sub_u8c4_f32c3, (p, w, h, pitch, sub_v, q, dpitch, _stream(stream)), defer)
+    return _deferred if defer else dst
 
 
-def divergent4_u8c4(src, gray_out, resized_out, mul_b, rect_c, mul_c, crop_out, sub_d, bgr_out, stream=None):
+def divergent4_u8c4(src, gray_out, resized_out, mul_b, rect_c, mul_c, crop_out, sub_d, bgr_out, stream=None, defer=False):
     """All four chains in one launch; outputs must be contiguous."""
     _, capi = load()
     p, w, h, pitch = _image(src, "uint8")
     for t in (gray_out, resized_out, crop_out, bgr_out):
         assert t.is_contiguous()
-    _check(capi.fk_divergent4_u8c4(p, w, h, pitch, C.c_void_p(_dev(gray_out, "uint8").data_ptr()), resized_out.shape[1],
+    _deferred = _call(capi.fk_divergent4_u8c4, (p, w, h, pitch, C.c_void_p(_dev(gray_out, "uint8").data_ptr()), resized_out.shape[1],
                                    resized_out.shape[0], mul_b, C.c_void_p(_dev(resized_out, "float32").data_ptr()),
                                    Rect(*rect_c), mul_c, C.c_void_p(_dev(crop_out, "uint8").data_ptr()), sub_d,
-                                   C.c_void_p(_dev(bgr_out, "float32").data_ptr()), _stream(stream)))
+                                   C.c_void_p(_dev(bgr_out, "float32").data_ptr()), _stream(stream)), defer)
+    return _deferred
 
 
-def batch_crop_cast_tensor(src, rects, out, stream=None):
+def batch_crop_cast_tensor(src, rects, out, stream=None, defer=False):
     """out: (n, max_h, max_w, 3) float32 contiguous; elements outside a plane's own rect stay untouched."""
     _, capi = load()
     p, w, h, pitch = _image(src, "uint8")
     out = _dev(out, "float32")
     n, mh, mw, _ = out.shape
     assert n == len(rects) and out.is_contiguous()
-    _check(capi.fk_batch_crop_cast_tensor(p, w, h, pitch, _rects(rects), n, mw, mh, C.c_void_p(out.data_ptr()), _stream(stream)))
-    return out
+    _deferred = _call(capi.fk_batch_crop_cast_tensor, (p, w, h, pitch, _rects(rects), n, mw, mh, C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out

@@ -188,7 +188,7 @@ struct PointwiseJob {
                                        : STAGE_OUT             ? OUT_BYTES
                                                                : 0;
     static constexpr int LDS_BYTES = BLOCK_THREADS * STAGE_BYTES;
-    static constexpr bool READ_IN_PLACE = N > 1 || sizeof(Prog) > 512; // run-time plane index, or a very long chain
+    static constexpr bool READ_IN_PLACE = N > 1 || sizeof(Prog) > 256; // run-time plane index, or a long chain (SGPR pressure)
     struct Plane {
         Prog prog;
         unsigned flags;
@@ -355,7 +355,6 @@ struct ResizeJob {
     // packed outputs whose four pixels per thread are not one 16-byte piece go out through LDS as whole 16-byte pieces
     static constexpr bool STAGE_OUT = !Out::IS_SPLIT && (RESIZE_PX * sizeof(OutPixel)) % 16 == 0 && RESIZE_PX * sizeof(OutPixel) > 16;
     static constexpr int OUT_STAGE_BYTES = STAGE_OUT ? RESIZE_TILE_H * OUT_ROW_BYTES : 0;
-    static constexpr int LDS_BYTES = (RESIZE_LDS_DWORDS * 4 > OUT_STAGE_BYTES ? RESIZE_LDS_DWORDS * 4 : OUT_STAGE_BYTES) + 16;
     static constexpr bool READ_IN_PLACE = N > 1;
     Prog plane[N];
     Out out;
@@ -540,7 +539,6 @@ struct ResizeJob {
 // ---- generic -----------------------------------------------------------------------------------------------------
 template <typename Sender, typename Receiver>
 struct GenericJob {
-    static constexpr int LDS_BYTES = 0;
     static constexpr bool READ_IN_PLACE = isBatchOperation<typename Sender::Operation>;
     Sender sender;
     Receiver receiver;

@@ -153,3 +153,30 @@ def test_argument_errors(fk, oracle):
         f = torch.zeros((4, 4, 3), device="cuda")
         fk.muladd_chain_f32c3(f, f.clone(), 3, 1.0, 1.0)
     torch.cuda.synchronize()
+
+
+def test_staged_parameter_block_path(oracle):
+    """Jobs above the kernel-argument limit are staged through device memory; force that with a tiny limit (the limit is
+    read once per process, hence the child process)."""
+    import os
+    import subprocess
+    import sys
+    code = (
+        "import numpy as np, torch, fusedkernellibrary_amd as fk\n"
+        "from oracle import binding as B\n"
+        "o = B.oracle(); rt, _ = fk.load(); assert rt.fkrt_max_kernarg_bytes() == 256\n"
+        "src = o.bytes(60, (200, 300, 3)); n = 32\n"
+        "rects = [((7 * i) % 200, (5 * i) % 120, 16 + (11 * i) % 80, 8 + (13 * i) % 70) for i in range(n)]\n"
+        "args = (B.PRESERVE_AR, (0, 0, 0), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)\n"
+        "want = o.crop_resize_muls_bgr_tensor(src, rects, (40, 24), *args)\n"
+        "out = torch.full((n, 24, 40, 3), float('nan'), device='cuda')\n"
+        "for _ in range(3): fk.crop_resize_muls_bgr_tensor(torch.from_numpy(src).cuda(), rects, out, *args)\n"
+        "torch.cuda.synchronize(); assert out.cpu().numpy().tobytes() == want.tobytes()\n"
+        "f = o.unit_floats(2, (64, 1024, 3)); d = torch.empty((64, 1024, 3), device='cuda')\n"
+        "fk.muladd_chain_f32c3(torch.from_numpy(f).cuda(), d, 64, 1.0001, 1e-4); torch.cuda.synchronize()\n"
+        "assert d.cpu().numpy().tobytes() == o.muladd_chain_f32c3(f, 64, 1.0001, 1e-4).tobytes()\n"
+        "print('staged ok')\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, FK_MAX_KERNARG_BYTES="256", PYTHONPATH=root)
+    proc = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=150)
+    assert proc.returncode == 0 and "staged ok" in proc.stdout, proc.stdout
