@@ -56,7 +56,7 @@ def build_cpp_tests():
     """The C++ programs under tests/cpp: the host-side API conformance check and the README example as user code."""
     tests = os.path.join(ROOT, "tests", "cpp")
     outs = []
-    for name in ("conformance", "readme_dropin"):
+    for name in ("conformance", "readme_dropin", "api_gpu"):
         out = os.path.join(tests, name)
         _run([hipcc(), "-x", "hip", os.path.join(tests, name + ".cpp"), "-I" + INCLUDE, *DEVICE_FLAGS, "-L" + HERE, "-lfk_hip_rt",
               "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/../../fusedkernellibrary_amd", "-o", out])

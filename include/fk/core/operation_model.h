@@ -727,8 +727,16 @@ private:
             return BatchRead<N, PlanePolicy::CONDITIONAL_WITH_DEFAULT>::build(
                 planes, cont.params.usedPlanes, detail::cast_channels<NewOutput>(cont.params.default_value));
         } else if constexpr (policyOf<SelfOp>() == PlanePolicy::CONDITIONAL_WITH_DEFAULT) {
-            return BatchRead<N, PlanePolicy::CONDITIONAL_WITH_DEFAULT>::build(
-                planes, self.params.usedPlanes, detail::cast_channels<NewOutput>(self.params.default_value));
+            if constexpr (isComputeType<ContIOp>) {
+                // the default value of the unused planes flows through the compute operation like any other value, as it
+                // does when the operation follows the batch read as a separate argument of executeOperations
+                return BatchRead<N, PlanePolicy::CONDITIONAL_WITH_DEFAULT>::build(
+                    planes, self.params.usedPlanes,
+                    detail::cast_channels<NewOutput>(compute(detail::cast_channels<GetInputType_t<ContIOp>>(self.params.default_value), cont)));
+            } else {
+                return BatchRead<N, PlanePolicy::CONDITIONAL_WITH_DEFAULT>::build(
+                    planes, self.params.usedPlanes, detail::cast_channels<NewOutput>(self.params.default_value));
+            }
         } else {
             return BatchRead<N, PlanePolicy::PROCESS_ALL>::build(planes);
         }

@@ -1,0 +1,141 @@
+// The rest of the executeOperations surface on the GPU, as user code: buffer overloads (fused_kernel.h:26-54 of the
+// reference), conditional batches with a default value (batch_operations.h:234-241), 1-D and 3-D reads (generic kernel),
+// cropped buffer views, the thread-fusion tag, setTo, stream sharing and error reporting.  Self-checking: exit code 0.
+#include <fused_kernel/fused_kernel.h>
+#include <fused_kernel/algorithms/image_processing/saturate.h>
+
+#include <cmath>
+#include <cstdio>
+
+using namespace fk;
+
+static int failures = 0;
+#define EXPECT(cond)                                                                                                   \
+    do {                                                                                                               \
+        if (!(cond)) {                                                                                                 \
+            std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);                                              \
+            ++failures;                                                                                                \
+        }                                                                                                              \
+    } while (0)
+
+template <typename T>
+static void fill_ramp(Ptr2D<T>& img, Stream& stream, int scale) {
+    const auto d = img.dims();
+    for (uint y = 0; y < d.height; ++y)
+        for (uint x = 0; x < d.width; ++x) img.at(x, y) = make_set<T>((x * 3 + y * 7) * scale % 251);
+    img.upload(stream);
+}
+
+int main() {
+    Stream stream;
+    Stream alias = stream; // copies share the native stream
+    EXPECT(alias.getHIPStream() == stream.getHIPStream() && stream.getRefCount() == 2);
+
+    // 1. conditional batch: planes >= activeBatch take the default value, then run through the same compute operations
+    {
+        constexpr size_t BATCH = 3;
+        std::array<Ptr2D<uchar3>, BATCH> inputs{ Ptr2D<uchar3>(16, 8), Ptr2D<uchar3>(16, 8), Ptr2D<uchar3>(16, 8) };
+        for (size_t i = 0; i < BATCH; ++i) setTo(uchar3{ static_cast<uchar>(10 * (i + 1)), 1, 2 }, inputs[i], stream);
+        Tensor<float3> out(16, 8, BATCH);
+        executeOperations<TransformDPP<>>(inputs, 2, uchar3{ 9, 9, 9 }, out, stream, Cast<uchar3, float3>::build(),
+                                          Mul<float3>::build(make_set<float3>(2.f)));
+        out.download(stream);
+        stream.sync();
+        bool ok = true;
+        for (uint y = 0; y < 8; ++y)
+            for (uint x = 0; x < 16; ++x) {
+                ok = ok && out.at(x, y, 0).x == 20.f && out.at(x, y, 0).z == 4.f && out.at(x, y, 1).x == 40.f && out.at(x, y, 2).x == 18.f &&
+                     out.at(x, y, 2).y == 18.f;
+            }
+        EXPECT(ok);
+    }
+    // 2. input / output buffer overload, scalar pixels (16 per thread), odd size and the runtime's padded pitch
+    {
+        Ptr2D<uchar> in(1237, 19);
+        Ptr2D<float> out(1237, 19);
+        fill_ramp(in, stream, 1);
+        executeOperations<TransformDPP<>>(in, out, stream, Cast<uchar, float>::build(), Add<float>::build(0.5f));
+        out.download(stream);
+        stream.sync();
+        bool ok = true;
+        for (uint y = 0; y < 19; ++y)
+            for (uint x = 0; x < 1237; ++x) ok = ok && out.at(x, y) == static_cast<float>(in.at(x, y)) + 0.5f;
+        EXPECT(ok);
+    }
+    // 3. 1-D buffers (generic kernel) under the thread-fusion tag
+    {
+        Ptr1D<float> in(1000), out(1000);
+        for (uint i = 0; i < 1000; ++i) in.at(i) = 0.25f * static_cast<float>(i);
+        Stream s2;
+        in.upload(s2);
+        executeOperations<TransformDPP<ParArch::GPU_AMD, TF::ENABLED>>(in, out, s2, Mul<float>::build(3.f), Sub<float>::build(1.f));
+        out.download(s2);
+        s2.sync();
+        bool ok = true;
+        for (uint i = 0; i < 1000; ++i) ok = ok && out.at(i) == 0.25f * static_cast<float>(i) * 3.f - 1.f;
+        EXPECT(ok);
+    }
+    // 4. 3-D read into a 3-D write, every plane (generic kernel), and getPlane views
+    {
+        Tensor<float> in(33, 5, 4), out(33, 5, 4);
+        for (uint z = 0; z < 4; ++z)
+            for (uint y = 0; y < 5; ++y)
+                for (uint x = 0; x < 33; ++x) in.at(x, y, z) = static_cast<float>(z * 1000 + y * 100 + x);
+        in.upload(stream);
+        executeOperations<TransformDPP<>>(stream, TensorRead<float>::build(in), Add<float>::build(1.f), TensorWrite<float>::build(out));
+        out.download(stream);
+        stream.sync();
+        bool ok = true;
+        for (uint z = 0; z < 4; ++z)
+            for (uint y = 0; y < 5; ++y)
+                for (uint x = 0; x < 33; ++x) ok = ok && out.at(x, y, z) == static_cast<float>(z * 1000 + y * 100 + x) + 1.f;
+        EXPECT(ok);
+        EXPECT(out.getPlane(2).at(7, 3) == 2000.f + 300.f + 7.f + 1.f);
+    }
+    // 5. a cropped view of a buffer as the source (unaligned base), SaturateCast and RGB2Gray
+    {
+        Ptr2D<float4> in(100, 40);
+        for (uint y = 0; y < 40; ++y)
+            for (uint x = 0; x < 100; ++x) in.at(x, y) = float4{ x * 3.f - 20.f, y * 7.f + 0.5f, 127.5f, 300.f };
+        in.upload(stream);
+        Ptr2D<float4> view = in.crop2D(Point(3, 2), PtrDims<ND::_2D>(61, 33));
+        Ptr2D<uchar4> out(61, 33);
+        executeOperations<TransformDPP<>>(view, out, stream, SaturateCast<float4, uchar4>::build());
+        out.download(stream);
+        stream.sync();
+        bool ok = true;
+        for (uint y = 0; y < 33; ++y)
+            for (uint x = 0; x < 61; ++x) {
+                const float fx = (x + 3) * 3.f - 20.f, fy = (y + 2) * 7.f + 0.5f;
+                const uchar4 v = out.at(x, y);
+                ok = ok && v.x == (fx < 0.f ? 0 : fx > 255.f ? 255 : static_cast<uchar>(fx)) &&
+                     v.y == (fy > 255.f ? 255 : static_cast<uchar>(fy + 0.5f)) && v.z == 128 && v.w == 255;
+            }
+        EXPECT(ok);
+        Ptr2D<uchar3> rgb(77, 9);
+        Ptr2D<uchar> gray(77, 9);
+        fill_ramp(rgb, stream, 5);
+        executeOperations<TransformDPP<>>(rgb, gray, stream, ColorConversion<ColorConversionCodes::COLOR_RGB2GRAY, uchar3, uchar>::build());
+        gray.download(stream);
+        stream.sync();
+        ok = true;
+        for (uint y = 0; y < 9; ++y)
+            for (uint x = 0; x < 77; ++x) {
+                const uchar3 p = rgb.at(x, y);
+                ok = ok && gray.at(x, y) == static_cast<uchar>(std::nearbyint((p.x * 0.299f + p.y * 0.587f) + p.z * 0.114f));
+            }
+        EXPECT(ok);
+    }
+    // 6. a launch the runtime rejects surfaces as the reference's exception text
+    {
+        bool threw = false;
+        try {
+            gpuErrchk(fkrt_launch(nullptr, 1, 1, 1, 256, 1, 1, nullptr, 0, stream));
+        } catch (const std::runtime_error& e) {
+            threw = std::string(e.what()).rfind("GPU Error: ", 0) == 0;
+        }
+        EXPECT(threw);
+    }
+    if (failures == 0) std::printf("api_gpu ok\n");
+    return failures == 0 ? 0 : 1;
+}

@@ -32,3 +32,11 @@ def test_readme_example_as_user_code(oracle, tmp_path):
     rects = [(0, 0, 34, 25), (10, 10, 70, 15), (20, 20, 60, 59), (30, 30, 20, 23), (40, 40, 12, 11)]
     want = oracle.crop_resize_muls_bgr_tensor(src, rects, (60, 60), B.PRESERVE_AR, (0, 0, 0), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)
     assert same_bits(got, want)
+
+
+@pytest.mark.gpu
+def test_executor_surface_as_user_code():
+    exe = os.path.join(HERE, "cpp", "api_gpu")
+    assert os.path.exists(exe), "tests/cpp/api_gpu is not built"
+    proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert proc.returncode == 0 and "api_gpu ok" in proc.stdout, proc.stdout
