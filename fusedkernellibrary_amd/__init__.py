@@ -67,10 +67,18 @@ def library_paths():
     return os.path.join(_HERE, "libfk_hip_rt.so"), os.path.join(_HERE, "libfk_capi.so")
 
 
+def use_literal_interpolation(enable=True):
+    """Switch the chain entry points to libfk_capi_literal.so, built with the reference's host-branch bilinear
+    interpolation (row index from the x coordinate).  For parity demonstrations against the reference CPU backend."""
+    _libs.pop("capi", None)
+    _libs["variant"] = "libfk_capi_literal.so" if enable else "libfk_capi.so"
+
+
 def load():
     """Load (once) and return (runtime, capi) ctypes handles; raises FkError when they have not been built."""
     if "capi" not in _libs:
         rt_path, capi_path = library_paths()
+        capi_path = os.path.join(_HERE, _libs.get("variant", "libfk_capi.so"))
         for p in (rt_path, capi_path):
             if not os.path.exists(p):
                 raise FkError(f"native library {p} is missing: build it with `python -m fusedkernellibrary_amd.build`")

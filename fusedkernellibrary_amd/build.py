@@ -64,8 +64,14 @@ def build_cpp_tests():
     return outs
 
 
+def build_literal_capi():
+    """The same chain entry points built with the reference's host-branch interpolation (bilinear row index taken from
+    the x coordinate): only there to show parity with the reference CPU backend's own output where that is defined."""
+    return build_capi(extra_defines=("FK_INTERPOLATE_Y1_FROM_X",), name="libfk_capi_literal.so")
+
+
 def build_all():
-    return [build_runtime(), build_capi()] + build_cpp_tests()
+    return [build_runtime(), build_capi(), build_literal_capi()] + build_cpp_tests()
 
 
 if __name__ == "__main__":

@@ -63,6 +63,11 @@ struct PlaneIOpOf<Sender, std::enable_if_t<isBatchOperation<typename Sender::Ope
     static constexpr bool process_all = Batch::PP == PlanePolicy::PROCESS_ALL;
     static type get(const Sender& s, size_t i) { return toIOp<typename Batch::Operation>(s.params.opData[i]); }
 };
+template <typename PlaneIOp, typename = void>
+struct IsResizeProgram : std::false_type {};
+template <typename PlaneIOp>
+struct IsResizeProgram<PlaneIOp, std::enable_if_t<ProgramOf<PlaneIOp>::supported>>
+    : std::bool_constant<ProgramOf<PlaneIOp>::View::IS_RESIZE> {};
 template <typename PlaneIOp, typename Receiver, typename = void>
 struct Matches : std::false_type {};
 template <typename PlaneIOp, typename Receiver>
@@ -75,7 +80,14 @@ struct JobOf {
     using Planes = detail::PlaneIOpOf<Sender>;
     using PlaneIOp = typename Planes::type;
     static constexpr size_t N = Planes::planes;
-    static constexpr bool viewable = Planes::process_all && detail::Matches<PlaneIOp, Receiver>::value;
+#ifdef FK_INTERPOLATE_Y1_FROM_X
+    // the reference's host-branch interpolation takes the tap row from the x coordinate: rows and columns are no longer
+    // separable, so resize chains run on the generic per-element kernel in such a build
+    static constexpr bool separable = !detail::IsResizeProgram<PlaneIOp>::value;
+#else
+    static constexpr bool separable = true;
+#endif
+    static constexpr bool viewable = Planes::process_all && separable && detail::Matches<PlaneIOp, Receiver>::value;
 
     static auto make(const Sender& sender, const Receiver& receiver) {
         if constexpr (viewable) {

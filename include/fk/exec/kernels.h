@@ -376,21 +376,21 @@ struct ResizeJob {
     }
 
     // Four consecutive pixels of row y, taps from the staged tile (STAGED) or straight from memory.
-    template <bool STAGED>
+    template <bool STAGED, bool INTERIOR>
     __device__ __attribute__((always_inline)) static inline void pixels(const Prog& prog, const unsigned int* tile, const char* window,
                                                                        int sx_lo, int sy_lo, int stride, int x_first, int y, OutPixel* o) {
         const View& v = prog.view;
         const PlainView<Src>& s = v.src;
         const int ry = y + v.off_y;
-        bool row_inside = y < v.h;
-        if constexpr (View::HAS_ROI) row_inside = row_inside && ry >= v.y1 && ry <= v.y2;
+        bool row_inside = INTERIOR || y < v.h;
+        if constexpr (View::HAS_ROI && !INTERIOR) row_inside = row_inside && ry >= v.y1 && ry <= v.y2;
         const float src_y = (ry - v.y1) * v.fy;
 #pragma unroll
         for (int k = 0; k < RESIZE_PX; ++k) {
             const int x = x_first + k;
             const int rx = x + v.off_x;
-            bool inside = row_inside && x < v.w;
-            if constexpr (View::HAS_ROI) inside = inside && rx >= v.x1 && rx <= v.x2;
+            bool inside = INTERIOR || (row_inside && x < v.w);
+            if constexpr (View::HAS_ROI && !INTERIOR) inside = inside && rx >= v.x1 && rx <= v.x2;
             Pixel value = v.background;
             if (inside) {
                 const float src_x = (rx - v.x1) * v.fx;
@@ -456,7 +456,6 @@ struct ResizeJob {
                                    static_cast<size_t>(s.ox) * sizeof(Src); // window pixel (0, 0)
         const int valid_lo = -s.ox * static_cast<int>(sizeof(Src));
         const int valid_hi = (s.img_w - s.ox) * static_cast<int>(sizeof(Src));
-#ifndef FK_INTERPOLATE_Y1_FROM_X
         if (resamples) {
             // source bounding box of the tile: taps are floor(c) and floor(c) + 1 for c in [lo, hi] * f; the column and
             // row past the source edge are staged as copies of the last one, which is what the clamp of the taps reads
@@ -482,15 +481,22 @@ struct ResizeJob {
                 }
             }
         }
-#endif
         dev::block_sync();
 
         // ---- this thread's four pixels; the tap source is decided once for the block ----
         OutPixel o[RESIZE_PX];
+        // interior tiles (whole tile inside the plane and inside the region that holds the image) need no per-pixel tests
+        bool interior = tx0 + RESIZE_TILE_W <= v.w && ty0 + RESIZE_TILE_H <= v.h;
+        if constexpr (View::HAS_ROI) {
+            interior = interior && tx0 + v.off_x >= v.x1 && tx0 + RESIZE_TILE_W - 1 + v.off_x <= v.x2 && ty0 + v.off_y >= v.y1 &&
+                       ty0 + RESIZE_TILE_H - 1 + v.off_y <= v.y2;
+        }
         if (staged) {
-            pixels<true>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
+            if (interior) pixels<true, true>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
+            else pixels<true, false>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
         } else {
-            pixels<false>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
+            if (interior) pixels<false, true>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
+            else pixels<false, false>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
         }
 
         // ---- write ----

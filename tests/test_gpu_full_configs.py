@@ -114,3 +114,46 @@ def test_c1_readme_matches_reference_vectors_where_defined(fk, oracle):
     crop = src[y:y + h, x:x + w, ::-1].astype(np.float32)
     expect = ((crop * np.float32(1.4)) - np.float32(0.5)) / np.float32(255.0)
     assert same_bits(got[2, :59], expect.astype(np.float32))
+
+
+def test_literal_build_reproduces_the_reference_cpu_backend(fk, oracle):
+    """libfk_capi_literal.so takes the bilinear row index from x like the reference's host branch: its GPU output must
+    equal the vectors written by the reference's own CPU backend, every element, for every chain with a resize."""
+    import json
+    import os
+    here = os.path.dirname(os.path.abspath(__file__))
+    gold = np.load(os.path.join(here, "golden", "reference_vectors.npz"))
+    cases = json.load(open(os.path.join(here, "golden", "reference_cases.json")))
+    fk.use_literal_interpolation(True)
+    try:
+        _, capi = fk.load()
+        assert capi.fk_interpolate_y1_from_x() == 1
+        c = cases["readme"]
+        src = dev(oracle.bytes(c["seed"], tuple(c["src"])))
+        for aspect in (0, 1, 2, 3):
+            out = torch.full((5, 60, 60, 3), float("nan"), device="cuda")
+            fk.crop_resize_muls_bgr_tensor(src, c["rects"], out, aspect, c["background"], c["mul"], c["sub"], c["div"])
+            torch.cuda.synchronize()
+            assert same_bits(out.cpu().numpy(), gold[f"readme_ar{aspect}"]), aspect
+        c = cases["split"]
+        srcs = [dev(oracle.bytes(c["seed"] + i, tuple(c["src"]))) for i in range(c["n"])]
+        out = torch.full((c["n"], 3, c["dst"][1], c["dst"][0]), float("nan"), device="cuda")
+        fk.batch_crop_resize_norm_split(srcs, c["rects"], out, c["div1"], c["sub"], c["div2"])
+        torch.cuda.synchronize()
+        assert same_bits(out.cpu().numpy(), gold["split"])
+        c = cases["tiles"]
+        src = dev(oracle.gradient_noise_u8c3(c["seed"], c["src"][1], c["src"][0]))
+        out = torch.full((len(c["rects"]), c["tile"][1], c["tile"][0], 3), float("nan"), device="cuda")
+        fk.resize_crop_tiles(src, c["resized"], c["rects"], out, c["mul"])
+        torch.cuda.synchronize()
+        assert same_bits(out.cpu().numpy(), gold["tiles"])
+        c = cases["divergent"]
+        src = dev(oracle.bytes(c["seed"], tuple(c["src"])))
+        out = torch.full((c["resized"][1], c["resized"][0], 4), float("nan"), device="cuda")
+        fk.resize_mul_u8c4_f32c4(src, out, c["mul_b"])
+        torch.cuda.synchronize()
+        assert same_bits(out.cpu().numpy(), gold["div_resized"])
+    finally:
+        fk.use_literal_interpolation(False)
+        _, capi = fk.load()
+        assert capi.fk_interpolate_y1_from_x() == 0
