@@ -78,14 +78,18 @@ def cpu_baseline(src_host, budget_s=10.0):
             "ms_per_pass": 1e3 * dt / passes, "host_cores_available": os.cpu_count()}
 
 
-def other_configs(fk, timer, steps, warmup):
-    """Per-config kernel time, output Gpixel/s and algorithmic GB/s for the remaining chains (device-random inputs)."""
+def other_configs(fk, timer, steps, warmup, only=None):
+    """Per-config kernel time, output Gpixel/s and algorithmic GB/s for the remaining chains (device-random inputs).
+    `only` restricts the run to the configs whose name starts with it (for counter collection on one kernel)."""
     import torch
     res = {}
     g = torch.Generator(device="cuda").manual_seed(0)
 
     def rnd_u8(*shape):
         return torch.randint(0, 256, shape, dtype=torch.uint8, device="cuda", generator=g)
+
+    def want(name):
+        return only is None or name.startswith(only)
 
     def record(name, ms, out_px, alg_bytes, note=None):
         res[name] = {"ms": ms, "gpixel_s": out_px / ms / 1e6, "alg_bytes": alg_bytes, "gb_s": alg_bytes / ms / 1e6,
@@ -98,37 +102,44 @@ def other_configs(fk, timer, steps, warmup):
     rects = [(0, 0, 34, 25), (10, 10, 70, 15), (20, 20, 60, 59), (30, 30, 20, 23), (40, 40, 12, 11)]
     out1 = torch.empty((5, 60, 60, 3), device="cuda")
     a1 = (0, (0, 0, 0), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)
-    call = fk.crop_resize_muls_bgr_tensor(img4k, rects, out1, *a1, defer=True)
-    ms = time_launches(timer, lambda i: call(), steps, warmup)
-    record("C1_readme_60x60x5", ms, 18000, sum(r[2] * r[3] for r in rects) * 3 + 18000 * 12, "launch-latency bound")
+    if want("C1_readme_60x60x5"):
+        call = fk.crop_resize_muls_bgr_tensor(img4k, rects, out1, *a1, defer=True)
+        ms = time_launches(timer, lambda i: call(), steps, warmup)
+        record("C1_readme_60x60x5", ms, 18000, sum(r[2] * r[3] for r in rects) * 3 + 18000 * 12, "launch-latency bound")
 
     # C1 scaled: same chain, 5 crops of 1024x768 -> 1920x1080 (bandwidth-sized)
-    rects_s = [(64 * i, 48 * i, 1024, 768) for i in range(5)]
-    out1s = [torch.empty((5, 1080, 1920, 3), device="cuda") for _ in range(3)]
-    calls = [fk.crop_resize_muls_bgr_tensor(img4k, rects_s, o, *a1, defer=True) for o in out1s]
-    ms = time_launches(timer, lambda i: calls[i % 3](), steps, warmup)
-    record("C1_scaled_5x1024x768_to_1920x1080", ms, 5 * 1920 * 1080, 5 * 1024 * 768 * 3 + 5 * 1920 * 1080 * 12)
+    if want("C1_scaled_5x1024x768_to_1920x1080"):
+        rects_s = [(64 * i, 48 * i, 1024, 768) for i in range(5)]
+        out1s = [torch.empty((5, 1080, 1920, 3), device="cuda") for _ in range(3)]
+        calls = [fk.crop_resize_muls_bgr_tensor(img4k, rects_s, o, *a1, defer=True) for o in out1s]
+        ms = time_launches(timer, lambda i: calls[i % 3](), steps, warmup)
+        record("C1_scaled_5x1024x768_to_1920x1080", ms, 5 * 1920 * 1080, 5 * 1024 * 768 * 3 + 5 * 1920 * 1080 * 12)
+        del out1s, calls
 
     # C3: 50 crops of 50 images -> 224x224x3x50 planar
-    imgs = [rnd_u8(1080, 1920, 3) for _ in range(50)]
-    ws = torch.randint(16, 513, (50,), generator=torch.Generator().manual_seed(3)).tolist()
-    hs = torch.randint(16, 513, (50,), generator=torch.Generator().manual_seed(4)).tolist()
-    rects3 = [((1920 - w) // 2, (1080 - h) // 3, w, h) for w, h in zip(ws, hs)]
-    out3 = torch.empty((50, 3, 224, 224), device="cuda")
-    a3 = ((255.,) * 3, (.485, .456, .406), (.229, .224, .225))
-    call3 = fk.batch_crop_resize_norm_split(imgs, rects3, out3, *a3, defer=True)
-    ms = time_launches(timer, lambda i: call3(), steps, warmup)
-    record("C3_batch50_224x224_split", ms, 50 * 224 * 224, 50 * 224 * 224 * 12 + sum(3 * r[2] * r[3] for r in rects3))
-    del imgs
+    if want("C3_batch50_224x224_split"):
+        imgs = [rnd_u8(1080, 1920, 3) for _ in range(50)]
+        ws = torch.randint(16, 513, (50,), generator=torch.Generator().manual_seed(3)).tolist()
+        hs = torch.randint(16, 513, (50,), generator=torch.Generator().manual_seed(4)).tolist()
+        rects3 = [((1920 - w) // 2, (1080 - h) // 3, w, h) for w, h in zip(ws, hs)]
+        out3 = torch.empty((50, 3, 224, 224), device="cuda")
+        a3 = ((255.,) * 3, (.485, .456, .406), (.229, .224, .225))
+        call3 = fk.batch_crop_resize_norm_split(imgs, rects3, out3, *a3, defer=True)
+        ms = time_launches(timer, lambda i: call3(), steps, warmup)
+        record("C3_batch50_224x224_split", ms, 50 * 224 * 224, 50 * 224 * 224 * 12 + sum(3 * r[2] * r[3] for r in rects3))
+        del imgs, call3
 
     # C4: resize 4K -> 1280x720, 32 tiles of 128x128
-    rects4 = [(160 * i, 180 * j, 128, 128) for j in range(4) for i in range(8)]
-    out4 = torch.empty((32, 128, 128, 3), device="cuda")
-    call4 = fk.resize_crop_tiles(img4k, (1280, 720), rects4, out4, (1 / 255.,) * 3, defer=True)
-    ms = time_launches(timer, lambda i: call4(), steps, warmup)
-    record("C4_resize_crop_32x128x128", ms, 32 * 128 * 128, 32 * 383 * 383 * 3 + 32 * 128 * 128 * 12)
+    if want("C4_resize_crop_32x128x128"):
+        rects4 = [(160 * i, 180 * j, 128, 128) for j in range(4) for i in range(8)]
+        out4 = torch.empty((32, 128, 128, 3), device="cuda")
+        call4 = fk.resize_crop_tiles(img4k, (1280, 720), rects4, out4, (1 / 255.,) * 3, defer=True)
+        ms = time_launches(timer, lambda i: call4(), steps, warmup)
+        record("C4_resize_crop_32x128x128", ms, 32 * 128 * 128, 32 * 383 * 383 * 3 + 32 * 128 * 128 * 12)
 
     # C5: four chains over one 8192x8192 uchar4 image in one launch
+    if not want("C5_divergent4_8192x8192"):
+        return res
     big = rnd_u8(8192, 8192, 4)
     gray = torch.empty((8192, 8192), dtype=torch.uint8, device="cuda")
     small = torch.empty((512, 512, 4), device="cuda")
@@ -149,6 +160,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the depth sweep and the other configs")
+    ap.add_argument("--only-config", default=None,
+                    help="run only the named secondary config (prefix of C1_readme, C1_scaled, C3, C4, C5) and print its figures: "
+                         "for rocprofv3 counter runs on one kernel")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run plain device copies of the same 99.5 MB image (torch copy kernel) before the timed "
                          "region, so that a counter run has a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -166,6 +180,10 @@ def main():
     torch.cuda.set_device(0)
     rt, _ = fk.load()
     timer = StreamTimer(rt, torch.cuda.current_stream().cuda_stream)
+
+    if args.only_config is not None:
+        print(json.dumps(other_configs(fk, timer, args.steps, args.warmup, only=args.only_config)))
+        return
 
     src_host = binding.oracle().unit_floats(2, (H, W, 3))
     sets = 3
