@@ -71,7 +71,15 @@ def build_literal_capi():
 
 
 def build_all():
-    return [build_runtime(), build_capi(), build_literal_capi()] + build_cpp_tests()
+    """Everything, the independent hipcc runs side by side (each is single-threaded)."""
+    from concurrent.futures import ThreadPoolExecutor
+    outs = [build_runtime()]  # the others link against it
+    with ThreadPoolExecutor(max_workers=3) as pool:
+        jobs = [pool.submit(build_capi), pool.submit(build_literal_capi), pool.submit(build_cpp_tests)]
+        for job in jobs:
+            res = job.result()
+            outs += res if isinstance(res, list) else [res]
+    return outs
 
 
 if __name__ == "__main__":

@@ -14,6 +14,17 @@ def pytest_configure(config):
 
 
 @pytest.fixture(scope="session")
+def native_build():
+    """The native libraries and C++ test programs: used as built; compiled here only when nothing has been built yet."""
+    import fusedkernellibrary_amd as lib
+    from fusedkernellibrary_amd import build
+    wanted = list(lib.library_paths()) + [os.path.join(ROOT, "tests", "cpp", n) for n in ("conformance", "readme_dropin", "api_gpu")]
+    if not all(os.path.exists(p) for p in wanted):
+        build.build_all()
+    return wanted
+
+
+@pytest.fixture(scope="session")
 def oracle():
     from oracle import binding
     return binding.oracle()

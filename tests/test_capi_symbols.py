@@ -17,7 +17,7 @@ def declared_functions(header):
 
 
 @pytest.fixture(scope="module")
-def libs():
+def libs(native_build):
     rt_path, capi_path = fk.library_paths()
     assert os.path.exists(rt_path) and os.path.exists(capi_path), "native libraries are not built (python -m fusedkernellibrary_amd.build)"
     rt = ctypes.CDLL(rt_path, mode=ctypes.RTLD_GLOBAL)

@@ -11,7 +11,7 @@ from oracle import binding as B
 HERE = os.path.dirname(os.path.abspath(__file__))
 
 
-def test_host_api_conformance():
+def test_host_api_conformance(native_build):
     exe = os.path.join(HERE, "cpp", "conformance")
     assert os.path.exists(exe), "tests/cpp/conformance is not built (python -m fusedkernellibrary_amd.build)"
     proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
