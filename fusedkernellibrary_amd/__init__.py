@@ -51,7 +51,15 @@ CAPI_SIGNATURES = {
     "fk_rgba2bgr_sub_u8c4_f32c3": [_vp, _i, _i, _sz, _f, _vp, _sz, _vp],
     "fk_divergent4_u8c4": [_vp, _i, _i, _sz, _vp, _i, _i, _f, _vp, Rect, _i, _vp, _f, _vp, _vp],
     "fk_batch_crop_cast_tensor": [_vp, _i, _i, _sz, _rp, _i, _i, _i, _vp, _vp],
+    "fk_read_yuv": [_i, _vp, _sz, _i, _i, _vp, _sz, _vp],
+    "fk_write_yuv": [_i, _vp, _sz, _i, _i, _vp, _sz, _vp],
+    "fk_yuv_to_rgb": [_i, _i, _i, _i, _i, _vp, _sz, _i, _i, _vp, _sz, _vp],
+    "fk_yuv_crop_resize_norm_split": [_i, _i, _i, _vp, _sz, _i, _i, Rect, _i, _i, _f, _vp, _vp],
 }
+# PixelFormat / ColorRange / ColorPrimitives values of include/fk_capi.h
+NV12, NV21, P010, P210, Y210, UYVY = 0, 1, 3, 6, 8, 10
+RANGE_LIMITED, RANGE_FULL = 0, 1
+BT601, BT709, BT2020 = 0, 1, 2
 RUNTIME_SYMBOLS = [
     "fkrt_device_count", "fkrt_set_device", "fkrt_get_device", "fkrt_stream_create", "fkrt_stream_destroy",
     "fkrt_stream_sync", "fkrt_malloc", "fkrt_malloc_pitch", "fkrt_free", "fkrt_malloc_host", "fkrt_free_host",
@@ -262,4 +270,68 @@ def batch_crop_cast_tensor(src, rects, out, stream=None, defer=False):
     n, mh, mw, _ = out.shape
     assert n == len(rects) and out.is_contiguous()
     _deferred = _call(capi.fk_batch_crop_cast_tensor, (p, w, h, pitch, _rects(rects), n, mw, mh, C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+# ---- YUV front-end: `raw` is the 2D buffer of base elements (uint8, or uint16/int16 for 10-bit formats) ------------
+
+def _raw(t, fmt):
+    import torch
+    if not t.is_cuda or t.dim() != 2 or t.stride(1) != 1:
+        raise FkError("a raw YUV image is a 2D GPU tensor with contiguous rows")
+    wide = fmt in (P010, P210, Y210)
+    if t.dtype not in ((torch.uint16, torch.int16) if wide else (torch.uint8,)):
+        raise FkError("raw YUV image has the wrong element type for its format")
+    return C.c_void_p(t.data_ptr()), t.stride(0) * t.element_size()
+
+
+def _pixels(t):
+    if not t.is_cuda or t.dim() != 3 or t.stride(2) != 1 or t.stride(1) != t.shape[2]:
+        raise FkError("pixels must be a (h, w, c) GPU tensor, contiguous along a row")
+    return C.c_void_p(t.data_ptr()), t.stride(0) * t.element_size()
+
+
+def read_yuv(fmt, raw, out, stream=None, defer=False):
+    """raw image -> out: (h, w, 3) {Y, U, V} pixels of the raw element type."""
+    _, capi = load()
+    p, pitch = _raw(raw, fmt)
+    q, out_pitch = _pixels(out)
+    h, w, _ = out.shape
+    _deferred = _call(capi.fk_read_yuv, (fmt, p, pitch, w, h, q, out_pitch, _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def write_yuv(fmt, pixels, raw, stream=None, defer=False):
+    """(h, w, 3) {Y, U, V} pixels -> raw image."""
+    _, capi = load()
+    p, pitch = _pixels(pixels)
+    q, raw_pitch = _raw(raw, fmt)
+    h, w, _ = pixels.shape
+    _deferred = _call(capi.fk_write_yuv, (fmt, p, pitch, w, h, q, raw_pitch, _stream(stream)), defer)
+    return _deferred if defer else raw
+
+
+def yuv_to_rgb(fmt, color_range, primaries, raw, out, stream=None, defer=False):
+    """raw image -> out: (h, w, 3 or 4) RGB[A] pixels, of the raw element type or float32."""
+    import torch
+    _, capi = load()
+    p, pitch = _raw(raw, fmt)
+    q, out_pitch = _pixels(out)
+    h, w, cn = out.shape
+    if cn not in (3, 4):
+        raise FkError("output pixels have 3 or 4 channels")
+    _deferred = _call(capi.fk_yuv_to_rgb, (fmt, color_range, primaries, int(cn == 4), int(out.dtype == torch.float32), p, pitch, w, h, q,
+                                           out_pitch, _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def yuv_crop_resize_norm_split(fmt, color_range, primaries, raw, size, crop, out, div_v, stream=None, defer=False):
+    """raw image of size = (w, h) -> RGB -> crop (x, y, w, h) -> resize -> / div_v -> out: (3, dst_h, dst_w) float32."""
+    _, capi = load()
+    p, pitch = _raw(raw, fmt)
+    out = _dev(out, "float32")
+    _, dh, dw = out.shape
+    assert out.is_contiguous()
+    _deferred = _call(capi.fk_yuv_crop_resize_norm_split, (fmt, color_range, primaries, p, pitch, size[0], size[1], Rect(*[int(v) for v in crop]),
+                                                           dw, dh, float(div_v), C.c_void_p(out.data_ptr()), _stream(stream)), defer)
     return _deferred if defer else out

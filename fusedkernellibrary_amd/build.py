@@ -1,8 +1,8 @@
 """Build recipe of the native libraries (hipcc, gfx950 only).
 
   libfk_hip_rt.so   the C runtime ABI of include/fk_hip_rt.h (csrc/fk_hip_rt.cpp)
-  libfk_capi.so     the chain entry points of include/fk_capi.h (csrc/fk_capi.hip), i.e. the fused kernels
-                    instantiated from the fk:: templates under include/fk/
+  libfk_capi.so     the chain entry points of include/fk_capi.h (csrc/fk_capi.hip, csrc/fk_capi_yuv.hip), i.e. the
+                    fused kernels instantiated from the fk:: templates under include/fk/
 
 Run as `python -m fusedkernellibrary_amd.build`; outputs land beside this file.
 """
@@ -43,12 +43,26 @@ def build_runtime():
     return out
 
 
+CAPI_SOURCES = ("fk_capi.hip", "fk_capi_yuv.hip")
+
+
 def build_capi(extra_defines=(), name="libfk_capi.so"):
+    """One object per source (compiled side by side), linked into one shared library."""
+    from concurrent.futures import ThreadPoolExecutor
     out = os.path.join(HERE, name)
-    cmd = [hipcc(), "-x", "hip", os.path.join(CSRC, "fk_capi.hip"), "-I" + INCLUDE, *DEVICE_FLAGS, "-fPIC", "-shared",
-           "-L" + HERE, "-lfk_hip_rt", "-Wl,-rpath,$ORIGIN", "-o", out]
-    cmd += ["-D" + d for d in extra_defines]
-    _run(cmd)
+    defines = ["-D" + d for d in extra_defines]
+    objdir = os.path.join(HERE, "csrc", ".obj_" + name.replace(".so", ""))
+    os.makedirs(objdir, exist_ok=True)
+
+    def compile_one(src):
+        obj = os.path.join(objdir, src.replace(".hip", ".o"))
+        _run([hipcc(), "-x", "hip", os.path.join(CSRC, src), "-I" + INCLUDE, *DEVICE_FLAGS, *defines, "-fPIC", "-c", "-o", obj])
+        return obj
+
+    with ThreadPoolExecutor(max_workers=len(CAPI_SOURCES)) as pool:
+        objs = list(pool.map(compile_one, CAPI_SOURCES))
+    _run([hipcc(), *objs, "--offload-arch=gfx950", "-fPIC", "-shared", "-L" + HERE, "-lfk_hip_rt", "-Wl,-rpath,$ORIGIN", "-o", out])
+    shutil.rmtree(objdir, ignore_errors=True)
     return out
 
 

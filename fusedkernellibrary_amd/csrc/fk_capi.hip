@@ -2,45 +2,20 @@
 // (PerThreadRead(...).then(...)..., TensorWrite) and hands it to executeOperations, which instantiates the fused
 // gfx950 kernel for that chain.  Compiled by hipcc into libfk_capi.so.
 #include <array>
-#include <exception>
-#include <string>
 
-#include "fk/fused_kernel.h"
-#include "fk_capi.h"
+#include "fk_capi_common.h"
 
 using namespace fk;
+using namespace fk_capi;
+
+namespace fk_capi {
+std::string& last_error() {
+    thread_local std::string text;
+    return text;
+}
+} // namespace fk_capi
 
 namespace {
-thread_local std::string g_last_error;
-
-template <typename F>
-int guarded(F&& body) {
-    try {
-        return body();
-    } catch (const std::exception& e) {
-        g_last_error = e.what();
-        return FK_ERR_RUNTIME;
-    }
-}
-int bad_argument(const char* what) {
-    g_last_error = what;
-    return FK_ERR_ARGUMENT;
-}
-int unsupported(const char* what) {
-    g_last_error = what;
-    return FK_ERR_UNSUPPORTED;
-}
-
-template <typename T>
-RawPtr<ND::_2D, T> view2d(const void* data, int w, int h, size_t pitch) {
-    return RawPtr<ND::_2D, T>{ const_cast<T*>(static_cast<const T*>(data)),
-                               PtrDims<ND::_2D>(static_cast<uint>(w), static_cast<uint>(h), static_cast<uint>(pitch)) };
-}
-template <typename T>
-RawPtr<ND::_3D, T> view3d(void* data, int w, int h, int planes, int color_planes) {
-    return RawPtr<ND::_3D, T>{ static_cast<T*>(data), PtrDims<ND::_3D>(static_cast<uint>(w), static_cast<uint>(h), static_cast<uint>(planes),
-                                                                       static_cast<uint>(color_planes), static_cast<uint>(sizeof(T) * w)) };
-}
 template <size_t N>
 std::array<Rect, N> rects_of(const fk_rect* r) {
     std::array<Rect, N> out;
@@ -178,7 +153,7 @@ void run_sequence(Stream& stream, const Sequence& seq) {
 
 extern "C" {
 
-const char* fk_last_error(void) { return g_last_error.c_str(); }
+const char* fk_last_error(void) { return last_error().c_str(); }
 
 int fk_interpolate_y1_from_x(void) {
 #ifdef FK_INTERPOLATE_Y1_FROM_X

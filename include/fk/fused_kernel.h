@@ -4,6 +4,7 @@
 #define FK_FUSED_KERNEL_H
 
 #include "fk/exec/executor.h"
+#include "fk/ops/yuv.h"
 
 namespace fk {
 

@@ -88,6 +88,37 @@ int fk_divergent4_u8c4(const void* src, int w, int h, size_t src_pitch, void* gr
 int fk_batch_crop_cast_tensor(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n,
                               int max_w, int max_h, float* out, void* stream);
 
+/* ---- YUV front-end ------------------------------------------------------------------------------------------
+ * A raw YUV image is ONE 2D allocation of base elements (uint8 for the 8-bit formats, uint16 with the sample in the
+ * high bits for the 10-bit ones), rows src_pitch bytes apart, as RawImage<PF> describes it
+ * (algorithms/image_processing/raw_image.h:108-114): NV12/NV21/P010 hold `height` luma rows then height/2 rows of
+ * interleaved chroma pairs, P210 `height` luma rows then `height` chroma rows, UYVY/Y210 2*width elements per row.
+ * width and height must be even.  Unpacked pixels are 3 (or 4) base elements, interleaved. */
+
+/* PixelFormat, raw_image.h:48 (the formats whose read compiles in the reference) */
+enum { FK_PF_NV12 = 0, FK_PF_NV21 = 1, FK_PF_P010 = 3, FK_PF_P210 = 6, FK_PF_Y210 = 8, FK_PF_UYVY = 10 };
+/* ColorRange and ColorPrimitives, raw_image.h:27-28.  A YCbCr -> RGB matrix exists for (FULL, BT601), (FULL, BT709),
+ * (LIMITED, BT709) and (FULL, BT2020) (algorithms/image_processing/color_conversion.h:137-171); any other pair
+ * returns FK_ERR_UNSUPPORTED. */
+enum { FK_RANGE_LIMITED = 0, FK_RANGE_FULL = 1 };
+enum { FK_BT601 = 0, FK_BT709 = 1, FK_BT2020 = 2 };
+
+/* ReadYUV<PF> -> PerThreadWrite<_2D, base3> (color_conversion.h:315-400): the {Y, U, V} of every pixel. */
+int fk_read_yuv(int format, const void* src, size_t src_pitch, int width, int height, void* dst, size_t dst_pitch, void* stream);
+/* PerThreadRead<_2D, base3> -> WriteYUV<PF> (color_conversion.h:402-513): {Y, U, V} pixels into a raw image; each
+ * chroma sample takes the value of the last pixel that the reference's host loop lets write it. */
+int fk_write_yuv(int format, const void* src, size_t src_pitch, int width, int height, void* dst, size_t dst_pitch, void* stream);
+/* ReadYUV<PF> -> ConvertYUVToRGB<PF, range, primaries, alpha, pixel> -> PerThreadWrite (color_conversion.h:250-310).
+ * pixel = base3/base4 (float_out = 0) or float3/float4 (float_out = 1); alpha appends the depth's maximum. */
+int fk_yuv_to_rgb(int format, int range, int primaries, int alpha, int float_out, const void* src, size_t src_pitch, int width,
+                  int height, void* dst, size_t dst_pitch, void* stream);
+/* The README's backwards-vertical-fusion example (README.md:155-163 of the reference): ReadYUV<PF> ->
+ * ConvertYUVToRGB<PF, range, primaries, false> -> Crop(crop) -> Resize<INTER_LINEAR>(dst_w x dst_h) ->
+ * Div<float3>(div_v) -> TensorSplit<float3>: dst receives 3 planes of dst_h x dst_w floats.  Only the YUV samples
+ * that the interpolation of the crop touches are read. */
+int fk_yuv_crop_resize_norm_split(int format, int range, int primaries, const void* src, size_t src_pitch, int width, int height,
+                                  fk_rect crop, int dst_w, int dst_h, float div_v, float* dst, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -2,7 +2,7 @@
 
 `oracle()` loads oracle/libfkoracle.so, the plain-C restatement of the reference's CPU executor
 (fk_oracle.c); `reference()` loads oracle/_ref/libfkref.so, the reference's own headers compiled for
-its CPU backend (ref_driver.cpp), or returns None when that build is absent.  Both are built by
+its CPU backend (ref_driver.cpp, plus ref_driver_yuv.cpp in libfkref_yuv.so), or returns None when that build is absent.  Both are built by
 oracle/Makefile.  Only tests, the smoke check and the CPU-baseline leg of the benchmark import this
 module; the shipped library never does.
 """
@@ -15,6 +15,13 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
 PRESERVE_AR, IGNORE_AR, PRESERVE_AR_RN_EVEN, PRESERVE_AR_LEFT = 0, 1, 2, 3
+# PixelFormat / ColorRange / ColorPrimitives values of the reference's raw_image.h
+NV12, NV21, P010, P210, Y210, UYVY = 0, 1, 3, 6, 8, 10
+YUV_FORMATS = {"NV12": NV12, "NV21": NV21, "P010": P010, "P210": P210, "Y210": Y210, "UYVY": UYVY}
+RANGE_LIMITED, RANGE_FULL = 0, 1
+BT601, BT709, BT2020 = 0, 1, 2
+# the (range, primaries) pairs for which the reference defines a YCbCr -> RGB matrix
+YUV_MATRICES = [(RANGE_FULL, BT601), (RANGE_FULL, BT709), (RANGE_LIMITED, BT709), (RANGE_FULL, BT2020)]
 
 
 class Rect(C.Structure):
@@ -75,10 +82,20 @@ def build(with_reference=True):
 class _Lib:
     """Thin numpy-facing wrapper; `ref=True` talks to the reference driver (literal host semantics)."""
 
-    def __init__(self, cdll, ref):
+    def __init__(self, cdll, ref, yuv_cdll=None):
         self.c = cdll
         self.ref = ref
+        self.yuv = yuv_cdll
         pre = "fkr_" if ref else "fko_"
+        if yuv_cdll is not None:
+            _v = C.c_void_p
+            for name, sig in {"read_yuv": [_i, _v, _sz, _i, _i, _v, _sz], "write_yuv": [_i, _v, _sz, _i, _i, _v, _sz],
+                              "yuv_to_rgb": [_i, _i, _i, _i, _i, _v, _sz, _i, _i, _v, _sz],
+                              "yuv_crop_resize_norm_split": [_i, _i, _i, _v, _sz, _i, _i, Rect, _i, _i, _f] +
+                                                            ([] if ref else [_i]) + [_v]}.items():
+                fn = getattr(yuv_cdll, pre + name)
+                fn.argtypes = sig
+                fn.restype = C.c_int
         for name, sig in _CHAIN_SIGS.items():
             fn = getattr(cdll, pre + name)
             sig = list(sig)
@@ -232,6 +249,51 @@ class _Lib:
         return out
 
 
+    # ---- YUV front-end: `raw` is the (data_h, data_w) buffer of base elements, row stride = pitch ----
+    @staticmethod
+    def yuv_data_shape(fmt, w, h):
+        """(rows, columns, dtype) of the buffer that holds a w x h image of this format."""
+        wf, hf, dt = {NV12: (1, 1.5, np.uint8), NV21: (1, 1.5, np.uint8), P010: (1, 1.5, np.uint16),
+                      P210: (1, 2, np.uint16), Y210: (2, 1, np.uint16), UYVY: (2, 1, np.uint8)}[fmt]
+        return int(h * hf), int(w * wf), dt
+
+    def _yuv_fn(self, name):
+        if self.yuv is None:
+            raise RuntimeError("the YUV checker library is not built")
+        return getattr(self.yuv, ("fkr_" if self.ref else "fko_") + name)
+
+    @staticmethod
+    def _check(rc):
+        if rc != 0:
+            raise ValueError("format or matrix not defined by the reference")
+
+    def read_yuv(self, fmt, raw, w, h):
+        out = np.empty((h, w, 3), raw.dtype)
+        self._check(self._yuv_fn("read_yuv")(fmt, _p(raw), raw.strides[0], w, h, _p(out), out.strides[0]))
+        return out
+
+    def write_yuv(self, fmt, pixels, fill=0):
+        h, w, _ = pixels.shape
+        rows, cols, dt = self.yuv_data_shape(fmt, w, h)
+        raw = np.full((rows, cols), fill, dt)
+        self._check(self._yuv_fn("write_yuv")(fmt, _p(pixels), pixels.strides[0], w, h, _p(raw), raw.strides[0]))
+        return raw
+
+    def yuv_to_rgb(self, fmt, rng, prim, alpha, float_out, raw, w, h):
+        out = np.empty((h, w, 4 if alpha else 3), np.float32 if float_out else raw.dtype)
+        self._check(self._yuv_fn("yuv_to_rgb")(fmt, rng, prim, int(alpha), int(float_out), _p(raw), raw.strides[0], w, h,
+                                                _p(out), out.strides[0]))
+        return out
+
+    def yuv_crop_resize_norm_split(self, fmt, rng, prim, raw, w, h, crop, dst, div_v, quirk=0):
+        out = np.empty((3, dst[1], dst[0]), np.float32)
+        args = [fmt, rng, prim, _p(raw), raw.strides[0], w, h, Rect(*crop), dst[0], dst[1], float(div_v)]
+        if not self.ref:
+            args.append(quirk)
+        self._check(self._yuv_fn("yuv_crop_resize_norm_split")(*args, _p(out)))
+        return out
+
+
 _cache = {}
 
 
@@ -240,7 +302,8 @@ def oracle():
         path = os.path.join(_HERE, "libfkoracle.so")
         if not os.path.exists(path):
             build(with_reference=False)
-        _cache["o"] = _Lib(C.CDLL(path), ref=False)
+        cdll = C.CDLL(path)
+        _cache["o"] = _Lib(cdll, ref=False, yuv_cdll=cdll)
     return _cache["o"]
 
 
@@ -248,5 +311,7 @@ def reference():
     """The reference-headers build, or None when oracle/_ref/libfkref.so has not been built."""
     if "r" not in _cache:
         path = os.path.join(_HERE, "_ref", "libfkref.so")
-        _cache["r"] = _Lib(C.CDLL(path), ref=True) if os.path.exists(path) else None
+        yuv_path = os.path.join(_HERE, "_ref", "libfkref_yuv.so")
+        yuv = C.CDLL(yuv_path) if os.path.exists(yuv_path) else None
+        _cache["r"] = _Lib(C.CDLL(path), ref=True, yuv_cdll=yuv) if os.path.exists(path) else None
     return _cache["r"]

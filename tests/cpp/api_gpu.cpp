@@ -126,7 +126,50 @@ int main() {
             }
         EXPECT(ok);
     }
-    // 6. a launch the runtime rejects surfaces as the reference's exception text
+    // 6. YUV images: an NV12 frame allocated by Image<PF>, read as {Y, U, V}, converted, and written back as UYVY
+    {
+        constexpr uint W = 64, H = 48;
+        Image<PixelFormat::NV12> nv12(W, H);
+        EXPECT(nv12.getData().dims().width == W && nv12.getData().dims().height == H + H / 2 && nv12.imageHeight() == H);
+        auto bytes = nv12.getData();
+        for (uint y = 0; y < H; ++y)
+            for (uint x = 0; x < W; ++x) bytes.at(x, y) = static_cast<uchar>((x + 2 * y) % 220 + 16);
+        for (uint y = 0; y < H / 2; ++y)
+            for (uint x = 0; x < W; x += 2) {
+                bytes.at(x, H + y) = static_cast<uchar>(100 + x / 2 + y);     // U
+                bytes.at(x + 1, H + y) = static_cast<uchar>(200 - x / 2 - y); // V
+            }
+        nv12.upload(stream);
+        EXPECT(nv12.readAt(Point(5, 7)).x == (5 + 14) % 220 + 16 && nv12.readAt(Point(5, 7)).y == 100 + 2 + 3 && nv12.readAt(Point(5, 7)).z == 200 - 2 - 3);
+
+        Ptr2D<uchar3> yuv(W, H);
+        Ptr2D<uchar4> rgba(W, H);
+        Image<PixelFormat::UYVY> uyvy(W, H);
+        const auto read = ReadYUV<PixelFormat::NV12>::build(nv12);
+        executeOperations<TransformDPP<>>(stream, read, PerThreadWrite<ND::_2D, uchar3>::build(yuv));
+        executeOperations<TransformDPP<>>(stream, read, ConvertYUVToRGB<PixelFormat::NV12, ColorRange::Full, ColorPrimitives::bt709, true>::build(),
+                                          PerThreadWrite<ND::_2D, uchar4>::build(rgba));
+        executeOperations<TransformDPP<>>(stream, read, WriteYUV<PixelFormat::UYVY>::build(uyvy));
+        yuv.download(stream);
+        rgba.download(stream);
+        uyvy.download(stream);
+        stream.sync();
+        bool ok = true;
+        for (uint y = 0; y < H; ++y)
+            for (uint x = 0; x < W; ++x) {
+                const uchar3 want = nv12.readAt(Point(static_cast<int>(x), static_cast<int>(y)));
+                const uchar3 got = yuv.at(x, y);
+                ok = ok && got.x == want.x && got.y == want.y && got.z == want.z;
+                const uchar4 host_rgba = ConvertYUVToRGB<PixelFormat::NV12, ColorRange::Full, ColorPrimitives::bt709, true>::exec(want);
+                const uchar4 dev_rgba = rgba.at(x, y);
+                ok = ok && dev_rgba.x == host_rgba.x && dev_rgba.y == host_rgba.y && dev_rgba.z == host_rgba.z && dev_rgba.w == 255;
+                // 4:2:2 keeps the chroma of even rows and of odd rows apart; NV12 gives both rows the same pair
+                const uchar3 back = uyvy.readAt(Point(static_cast<int>(x), static_cast<int>(y)));
+                ok = ok && back.x == want.x && back.y == want.y && back.z == want.z;
+            }
+        EXPECT(ok);
+    }
+    // 7. a launch the runtime rejects surfaces as the reference's exception text
     {
         bool threw = false;
         try {

@@ -106,6 +106,32 @@ static_assert(kCondResized.params.usedPlanes == 2 && kCondResized.params.default
 constexpr std::array<Read<ReadU3>, 3> kThreeReads{ kRead, kRead, kRead };
 static_assert(std::decay_t<decltype(Resize<InterpolationType::INTER_LINEAR>::build(kThreeReads, kSizes))>::Operation::BATCH == 3);
 
+// YUV front-end: a YUV read fused with its conversion is a Read that Resize accepts as its back operation, and the
+// parameters of operations fused after it stay reachable (tests/operation/test_fused_operation.h:43-50 of the reference)
+constexpr auto kReadYUV = ReadYUV<PixelFormat::NV12>::build({ { RawPtr<ND::_2D, uchar>{ nullptr, PtrDims<ND::_2D>(128, 128 + 64) }, 128, 128 } });
+constexpr auto kReadRGB = kReadYUV.then(ConvertYUVToRGB<PixelFormat::NV12, ColorRange::Full, ColorPrimitives::bt2020, false>::build());
+static_assert(isReadType<std::decay_t<decltype(kReadRGB)>> && std::is_same_v<std::decay_t<decltype(kReadRGB)>::Operation::OutputType, uchar3>);
+constexpr auto kYUVResized = Resize<InterpolationType::INTER_LINEAR>::build(kReadRGB, Size(64, 64));
+constexpr auto kYUVResizedDiv = kYUVResized.then(Mul<float>::build(3.f)).then(Div<float>::build(4.3f));
+static_assert(kYUVResizedDiv.params.next.next.instance.params == 4.3f && kYUVResized.getActiveThreads() == ActiveThreads(64, 64, 1));
+static_assert(kYUVResized.params.params.src_size.width == 128 && kYUVResized.params.src_conv_factors.x == 2.f);
+// traits of the formats (raw_image.h:48-106; utest_color_conversion.h UYVY traits test of the reference)
+static_assert(PixelFormatTraits<PixelFormat::UYVY>::space == ColorSpace::YUV422 && PixelFormatTraits<PixelFormat::UYVY>::depth == ColorDepth::p8bit &&
+              PixelFormatTraits<PixelFormat::UYVY>::cn == 3 && PixelFormatTraits<PixelFormat::UYVY>::rf.width_f == 2.f);
+static_assert(std::is_same_v<RawImage<PixelFormat::P010>::BaseType, ushort> && std::is_same_v<ReadYUV<PixelFormat::Y210>::OutputType, ushort3> &&
+              std::is_same_v<YUVOutputPixelType<PixelFormat::NV21, true>, uchar4>);
+static_assert(IsEven<int>::exec(4) && !IsEven<uint>::exec(7u) && IsEven<int>::exec(-2) && !IsEven<int>::exec(-1));
+static_assert(ShiftRight<ushort3>::exec(ushort3{ 0xFFC0, 64, 63 }, 6).x == 1023 && ShiftLeft<ushort>::exec(1023, 6) == 0xFFC0 &&
+              ShiftLeft<ushort>::exec(0xFFFF, 6) == 0xFFC0, "shifts stay in the storage type");
+// studio-range grey through the bt601 matrix: (126 - 16) * 1.164383562 = 128.08 -> 128
+static_assert(ConvertYUVToRGB<PixelFormat::NV12, ColorRange::Full, ColorPrimitives::bt601, true>::exec(uchar3{ 126, 128, 128 }).x == 128 &&
+              ConvertYUVToRGB<PixelFormat::NV12, ColorRange::Full, ColorPrimitives::bt601, true>::exec(uchar3{ 126, 128, 128 }).w == 255);
+static_assert(ConvertYUVToRGB<PixelFormat::P010, ColorRange::Full, ColorPrimitives::bt709, true>::exec(ushort3{ 500 << 6, 512 << 6, 512 << 6 }).y == (500 << 6) &&
+              ConvertYUVToRGB<PixelFormat::P010, ColorRange::Full, ColorPrimitives::bt709, true>::exec(ushort3{ 500 << 6, 512 << 6, 512 << 6 }).w == (1023 << 6));
+static_assert(NormalizeColorRangeDepth<float3, ColorDepth::p8bit>::exec(float3{ 0.f, 128.f, 255.f }).z == 255.f &&
+              SaturateDenormalizePixel<float3, uchar3, ColorDepth::p8bit>::exec(float3{ -0.5f, 0.5f, 1.5f }).y == 127 &&
+              SaturateDenormalizePixel<float3, uchar3, ColorDepth::p8bit>::exec(float3{ -0.5f, 0.5f, 1.5f }).z == 255);
+
 // DPP tags
 static_assert(TransformDPP<>::PAR_ARCH == ParArch::GPU_AMD && defaultParArch == ParArch::GPU_AMD && Stream::parArch() == ParArch::GPU_AMD);
 static_assert(exec::pixels_per_thread<float3, float3, false>() == 4 && exec::pixels_per_thread<uchar4, uchar, false>() == 4 &&
