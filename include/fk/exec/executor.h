@@ -121,26 +121,26 @@ struct JobOf {
             } else {
                 using Job = PointwiseJob<Prog, N, Out>;
                 using Src = typename Job::Src;
+                using Access = typename Job::Access;
                 Job job{};
                 job.out = out;
-                constexpr size_t in_chunk = dev::chunk_bytes(Job::K * static_cast<int>(sizeof(Src)));
                 constexpr size_t out_elem = Out::IS_SPLIT ? sizeof(VBase<typename Out::Pixel>) : sizeof(typename Out::Pixel);
                 constexpr size_t out_chunk = dev::chunk_bytes(Job::K * static_cast<int>(out_elem));
                 int max_w = 0, max_h = 0;
                 for (size_t i = 0; i < N; ++i) {
                     job.plane[i].prog = ProgramOf<PlaneIOp>::make(Planes::get(sender, i));
                     auto& v = job.plane[i].prog.view;
-                    if (N == 1 && v.ox == 0 && v.oy == 0 && v.w == v.img_w && v.h > 1 &&
-                        v.pitch == static_cast<uint>(v.w) * sizeof(Src) && out.pitch == static_cast<uint>(v.w) * out_elem &&
-                        static_cast<size_t>(v.w) * v.h < (1u << 30)) {
-                        // rows are contiguous on both sides: treat the image as one long row, so no block is cut
-                        // short at a row end
-                        v.w = v.img_w = v.w * v.h;
-                        v.h = v.img_h = 1;
+                    if constexpr (Access::FLATTENS) {
+                        if (N == 1 && v.ox == 0 && v.oy == 0 && v.w == v.img_w && v.h > 1 &&
+                            v.pitch == static_cast<uint>(v.w) * sizeof(Src) && out.pitch == static_cast<uint>(v.w) * out_elem &&
+                            static_cast<size_t>(v.w) * v.h < (1u << 30)) {
+                            // rows are contiguous on both sides: treat the image as one long row, so no block is cut
+                            // short at a row end
+                            v.w = v.img_w = v.w * v.h;
+                            v.h = v.img_h = 1;
+                        }
                     }
-                    const char* const first = reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy) * v.pitch +
-                                              static_cast<size_t>(v.ox) * sizeof(Src);
-                    bool vec = aligned_to(first, in_chunk) && (v.h == 1 || v.pitch % in_chunk == 0);
+                    bool vec = Access::template aligned<Job::K>(v);
                     const char* const ofirst = reinterpret_cast<const char*>(out.data) + i * out.z_stride;
                     vec = vec && aligned_to(ofirst, out_chunk) && (v.h == 1 || out.pitch % out_chunk == 0);
                     if constexpr (Out::IS_SPLIT) vec = vec && out.chan_stride % out_chunk == 0;

@@ -1,11 +1,13 @@
 // The fused Transform kernels for gfx950 (CDNA4, wave64), hand-written against the views of fk/exec/views.h.
 //
 // Every launch runs blocks of 256 threads (four wave64).  A "job" is one fused chain over all its planes:
-//   PointwiseJob  element-wise chains over a PlainView: each thread owns K consecutive pixels of a row so that both the
-//                 source and the destination bytes of a thread are whole 16-byte (or 8/4-byte) transactions;
+//   PointwiseJob  element-wise chains over a PlainView or a YuvView: each thread owns K consecutive pixels of a row so
+//                 that both the source and the destination bytes of a thread are whole 16-byte (or 8/4-byte)
+//                 transactions (a YUV thread loads its luma run and the chroma pairs that cover it);
 //   ResizeJob     bilinear resize (with optional inner/outer crop and aspect-ratio border): a block owns a 64x16 output
 //                 tile, four pixels per thread; it stages the source bounding box of the tile in LDS, one dword-aligned
-//                 slot per source pixel, and takes the 2x2 taps from there; tiles that gain nothing from it (strong
+//                 slot per source pixel (after the operations fused before the resize, e.g. YUV -> RGB, so those run
+//                 once per source pixel), and takes the 2x2 taps from there; tiles that gain nothing from it (strong
 //                 down-scaling, no tap reuse) read their taps straight from memory; packed outputs leave through LDS
 //                 as whole 16-byte pieces;
 //   GenericJob    one thread per output element through Operation::exec, for any chain the views cannot describe.
@@ -167,21 +169,114 @@ constexpr int pixels_per_thread() {
     return 16;
 }
 
+// ---- source access -----------------------------------------------------------------------------------------------
+// SourceAccess<View>: one pixel of the window (load_one), K consecutive pixels of a row with vector loads (load_group,
+// when the host found the alignment that needs: `aligned`), and the pixels per thread that suit an output pixel type.
+template <typename View>
+struct SourceAccess;
+
+template <typename T>
+struct SourceAccess<PlainView<T>> {
+    using View = PlainView<T>;
+    static constexpr bool FLATTENS = true; // contiguous rows may be treated as one long row
+    template <typename O, bool SPLIT>
+    static constexpr int pixels() { return pixels_per_thread<T, O, SPLIT>(); }
+    template <int K>
+    static constexpr int group_bytes() { return K * static_cast<int>(sizeof(T)); }
+    __device__ __attribute__((always_inline)) static inline const char* row(const View& v, int y) {
+        return reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy + y) * v.pitch + static_cast<size_t>(v.ox) * sizeof(T);
+    }
+    __device__ __attribute__((always_inline)) static inline T load_one(const View& v, int x, int y) { return reinterpret_cast<const T*>(row(v, y))[x]; }
+    template <int K>
+    __device__ __attribute__((always_inline)) static inline void load_group(const View& v, int x0, int y, T* out) {
+        constexpr int NB = K * static_cast<int>(sizeof(T));
+        unsigned int w[NB / 4];
+        dev::load_words<NB>(row(v, y) + static_cast<size_t>(x0) * sizeof(T), w);
+        __builtin_memcpy(out, w, NB);
+    }
+    template <int K>
+    static bool aligned(const View& v) {
+        constexpr size_t chunk = dev::chunk_bytes(K * static_cast<int>(sizeof(T)));
+        const size_t first = reinterpret_cast<size_t>(v.data) + static_cast<size_t>(v.oy) * v.pitch + static_cast<size_t>(v.ox) * sizeof(T);
+        return first % chunk == 0 && (v.h == 1 || v.pitch % chunk == 0);
+    }
+};
+
+template <PixelFormat PF>
+struct SourceAccess<YuvView<PF>> {
+    using View = YuvView<PF>;
+    using Base = typename View::Base;
+    using Pixel = typename View::Pixel;
+    using Layout = fk::detail::YuvLayout<PF>;
+    static constexpr bool FLATTENS = false;
+    // smallest power of two >= 4 whose output run is whole 16-byte pieces and whose luma run is whole dwords
+    template <typename O, bool SPLIT>
+    static constexpr int pixels() {
+        const int so = SPLIT ? static_cast<int>(sizeof(VBase<O>)) : static_cast<int>(sizeof(O));
+        for (int k = 4; k <= 16; k *= 2) {
+            if ((k * so) % 16 == 0 && (k * static_cast<int>(sizeof(Base))) % 4 == 0) return k;
+        }
+        return 16;
+    }
+    // bytes of the widest single run a thread loads: K luma samples, or 2K packed samples
+    template <int K>
+    static constexpr int group_bytes() { return (Layout::semi_planar ? K : 2 * K) * static_cast<int>(sizeof(Base)); }
+    __device__ __attribute__((always_inline)) static inline Pixel load_one(const View& v, int x, int y) {
+        const RawImage<PF> raw{ RawPtr<ND::_2D, Base>{ const_cast<Base*>(v.data), PtrDims<ND::_2D>(0u, 0u, v.pitch) }, static_cast<uint>(v.img_w),
+                                static_cast<uint>(v.img_h) };
+        return ReadYUV<PF>::exec(Point(v.ox + x, v.oy + y), raw);
+    }
+    // x0 and v.ox are even: the K pixels are K/2 whole chroma pairs
+    template <int K>
+    __device__ __attribute__((always_inline)) static inline void load_group(const View& v, int x0, int y, Pixel* out) {
+        const int px = v.ox + x0, py = v.oy + y;
+        constexpr int NB = group_bytes<K>();
+        if constexpr (Layout::semi_planar) {
+            const char* const base = reinterpret_cast<const char*>(v.data);
+            unsigned int wl[NB / 4], wc[NB / 4];
+            dev::load_words<NB>(base + static_cast<size_t>(py) * v.pitch + static_cast<size_t>(px) * sizeof(Base), wl);
+            dev::load_words<NB>(base + (static_cast<size_t>(v.img_h) + (py >> Layout::row_shift)) * v.pitch + static_cast<size_t>(px) * sizeof(Base), wc);
+            Base luma[K], chroma[K];
+            __builtin_memcpy(luma, wl, NB);
+            __builtin_memcpy(chroma, wc, NB);
+#pragma unroll
+            for (int k = 0; k < K; ++k) out[k] = Pixel{ luma[k], chroma[(k & ~1) + Layout::u], chroma[(k & ~1) + Layout::v] };
+        } else {
+            unsigned int w[NB / 4];
+            dev::load_words<NB>(reinterpret_cast<const char*>(v.data) + static_cast<size_t>(py) * v.pitch + 2 * static_cast<size_t>(px) * sizeof(Base), w);
+            Base quad[2 * K];
+            __builtin_memcpy(quad, w, NB);
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                const int q = 4 * (k >> 1);
+                out[k] = Pixel{ quad[q + ((k & 1) ? Layout::y1 : Layout::y0)], quad[q + Layout::u], quad[q + Layout::v] };
+            }
+        }
+    }
+    template <int K>
+    static bool aligned(const View& v) {
+        constexpr size_t chunk = dev::chunk_bytes(group_bytes<K>());
+        const size_t first = reinterpret_cast<size_t>(v.data) + (Layout::semi_planar ? 1 : 2) * static_cast<size_t>(v.ox) * sizeof(Base);
+        return (v.ox & 1) == 0 && first % chunk == 0 && v.pitch % chunk == 0;
+    }
+};
+
 // ---- pointwise ---------------------------------------------------------------------------------------------------
 enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_STAGE_OUT = 8u };
 
 template <typename Prog, size_t N, typename Out>
 struct PointwiseJob {
     using View = decltype(Prog::view);
+    using Access = SourceAccess<View>;
     using Src = typename View::Source;
     using OutPixel = typename Out::Pixel;
-    static constexpr int K = pixels_per_thread<Src, OutPixel, Out::IS_SPLIT>();
+    static constexpr int K = Access::template pixels<OutPixel, Out::IS_SPLIT>();
     static constexpr int IN_BYTES = K * static_cast<int>(sizeof(Src));
     static constexpr int OUT_BYTES = Out::IS_SPLIT ? K * static_cast<int>(sizeof(VBase<OutPixel>)) : K * static_cast<int>(sizeof(OutPixel));
     // A thread's K pixels span more than one 16-byte transaction when pixels are 12 bytes wide (48 bytes per thread).
-    // Lanes reading 48-byte runs touch every cache line three times; instead the block moves its contiguous
-    // 256*K-pixel span with fully coalesced 16-byte accesses and redistributes pixels to threads through LDS.
-    static constexpr bool STAGE_IN = IN_BYTES > 16 && IN_BYTES % 16 == 0;
+    // Lanes reading 48-byte runs touch every cache line three times; instead the block moves its contiguous span of up
+    // to 256*K pixels with fully coalesced 16-byte accesses and redistributes pixels to threads through LDS.
+    static constexpr bool STAGE_IN = Access::FLATTENS && IN_BYTES > 16 && IN_BYTES % 16 == 0;
     static constexpr bool STAGE_OUT = !Out::IS_SPLIT && OUT_BYTES > 16 && OUT_BYTES % 16 == 0;
     static constexpr int STAGE_BYTES = (STAGE_IN && STAGE_OUT) ? (IN_BYTES > OUT_BYTES ? IN_BYTES : OUT_BYTES)
                                        : STAGE_IN              ? IN_BYTES
@@ -208,52 +303,62 @@ struct PointwiseJob {
         const int y = static_cast<int>(by) * (BLOCK_THREADS >> job.tx_shift) + (tid >> job.tx_shift);
 
         if constexpr (STAGE_IN || STAGE_OUT) {
-            // block-uniform: the whole block lies on one row and its 256*K pixels are all inside the plane
-            const bool whole = (pl.flags & FLAG_VECTOR_IO) != 0u && job.tx_shift == 8u && y < v.h &&
-                               (static_cast<int>(bx) + 1) * BLOCK_THREADS * K <= v.w;
-            if (whole) {
-                const int bx0 = static_cast<int>(bx) * BLOCK_THREADS * K; // first pixel of the block
+            // block-uniform: the whole block lies on one row; `span` pixels of that row are the block's, a whole number
+            // of thread groups, so the span is whole 16-byte pieces on both sides
+            const int bx0 = static_cast<int>(bx) * BLOCK_THREADS * K; // first pixel of the block
+            const int span = v.w - bx0 < BLOCK_THREADS * K ? v.w - bx0 : BLOCK_THREADS * K;
+            const bool rowwise = (pl.flags & FLAG_VECTOR_IO) != 0u && job.tx_shift == 8u && y < v.h && span > 0 && span % K == 0;
+            if (rowwise) {
                 dev::u32x4* const stage = reinterpret_cast<dev::u32x4*>(lds);
+                const bool active = x0 < v.w;
                 Src in[K];
                 if constexpr (STAGE_IN) {
-                    const dev::u32x4* const g = reinterpret_cast<const dev::u32x4*>(
-                        reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy + y) * v.pitch +
-                        static_cast<size_t>(v.ox + bx0) * sizeof(Src));
+                    const dev::u32x4* const g = reinterpret_cast<const dev::u32x4*>(Access::row(v, y) + static_cast<size_t>(bx0) * sizeof(Src));
+                    const int pieces = span * static_cast<int>(sizeof(Src)) / 16;
 #pragma unroll
-                    for (int j = 0; j < IN_BYTES / 16; ++j) stage[j * BLOCK_THREADS + tid] = g[j * BLOCK_THREADS + tid];
+                    for (int j = 0; j < IN_BYTES / 16; ++j) {
+                        if (j * BLOCK_THREADS + tid < pieces) stage[j * BLOCK_THREADS + tid] = g[j * BLOCK_THREADS + tid];
+                    }
                     dev::block_sync();
-                    dev::u32x4 mine[IN_BYTES / 16];
+                    if (active) {
+                        dev::u32x4 mine[IN_BYTES / 16];
 #pragma unroll
-                    for (int j = 0; j < IN_BYTES / 16; ++j) mine[j] = stage[tid * (IN_BYTES / 16) + j];
-                    __builtin_memcpy(in, mine, IN_BYTES);
+                        for (int j = 0; j < IN_BYTES / 16; ++j) mine[j] = stage[tid * (IN_BYTES / 16) + j];
+                        __builtin_memcpy(in, mine, IN_BYTES);
+                    }
                 } else {
-                    const char* const srow = reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy + y) * v.pitch +
-                                             static_cast<size_t>(v.ox) * sizeof(Src);
-                    unsigned int w[IN_BYTES / 4];
-                    dev::load_words<IN_BYTES>(srow + static_cast<size_t>(x0) * sizeof(Src), w);
-                    __builtin_memcpy(in, w, IN_BYTES);
+                    if (active) Access::template load_group<K>(v, x0, y, in);
                 }
                 OutPixel o[K];
+                if (active) {
 #pragma unroll
-                for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
+                    for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
+                }
                 if constexpr (STAGE_OUT) {
                     if constexpr (STAGE_IN) dev::block_sync(); // every thread has taken its input out of the buffer
-                    dev::u32x4 mine[OUT_BYTES / 16];
-                    __builtin_memcpy(mine, o, OUT_BYTES);
+                    if (active) {
+                        dev::u32x4 mine[OUT_BYTES / 16];
+                        __builtin_memcpy(mine, o, OUT_BYTES);
 #pragma unroll
-                    for (int j = 0; j < OUT_BYTES / 16; ++j) stage[tid * (OUT_BYTES / 16) + j] = mine[j];
+                        for (int j = 0; j < OUT_BYTES / 16; ++j) stage[tid * (OUT_BYTES / 16) + j] = mine[j];
+                    }
                     dev::block_sync();
                     dev::u32x4* const g = reinterpret_cast<dev::u32x4*>(
                         reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
                         static_cast<size_t>(y) * job.out.pitch + static_cast<size_t>(bx0) * sizeof(OutPixel));
+                    const int pieces = span * static_cast<int>(sizeof(OutPixel)) / 16;
                     if ((pl.flags & FLAG_STREAM_STORES) != 0u) {
 #pragma unroll
-                        for (int j = 0; j < OUT_BYTES / 16; ++j) dev::store_piece<true>(g + j * BLOCK_THREADS + tid, stage[j * BLOCK_THREADS + tid]);
+                        for (int j = 0; j < OUT_BYTES / 16; ++j) {
+                            if (j * BLOCK_THREADS + tid < pieces) dev::store_piece<true>(g + j * BLOCK_THREADS + tid, stage[j * BLOCK_THREADS + tid]);
+                        }
                     } else {
 #pragma unroll
-                        for (int j = 0; j < OUT_BYTES / 16; ++j) g[j * BLOCK_THREADS + tid] = stage[j * BLOCK_THREADS + tid];
+                        for (int j = 0; j < OUT_BYTES / 16; ++j) {
+                            if (j * BLOCK_THREADS + tid < pieces) g[j * BLOCK_THREADS + tid] = stage[j * BLOCK_THREADS + tid];
+                        }
                     }
-                } else {
+                } else if (active) {
                     if ((pl.flags & FLAG_STREAM_STORES) != 0u) dev::store_group<K, true>(job.out, x0, y, static_cast<int>(bz), o);
                     else dev::store_group<K>(job.out, x0, y, static_cast<int>(bz), o);
                 }
@@ -262,13 +367,9 @@ struct PointwiseJob {
         }
 
         if (y >= v.h || x0 >= v.w) return; // also ends blocks that lie outside a smaller plane of a ragged batch
-        const char* const srow = reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy + y) * v.pitch +
-                                 static_cast<size_t>(v.ox) * sizeof(Src);
         if ((pl.flags & FLAG_VECTOR_IO) != 0u && x0 + K <= v.w) {
-            unsigned int w[IN_BYTES / 4];
-            dev::load_words<IN_BYTES>(srow + static_cast<size_t>(x0) * sizeof(Src), w);
             Src in[K];
-            __builtin_memcpy(in, w, IN_BYTES);
+            Access::template load_group<K>(v, x0, y, in);
             OutPixel o[K];
 #pragma unroll
             for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
@@ -277,7 +378,7 @@ struct PointwiseJob {
         } else {
             const int xe = x0 + K < v.w ? x0 + K : v.w;
             for (int x = x0; x < xe; ++x) {
-                const OutPixel o = dev::apply_tail(pl.prog.tail, reinterpret_cast<const Src*>(srow)[x]);
+                const OutPixel o = dev::apply_tail(pl.prog.tail, Access::load_one(v, x, y));
                 dev::store_one(job.out, x, y, static_cast<int>(bz), o);
             }
         }
@@ -347,9 +448,14 @@ __device__ __attribute__((always_inline)) inline PixelSlot<T> load_pixel_slot(co
 template <typename Prog, size_t N, typename Out>
 struct ResizeJob {
     using View = decltype(Prog::view);
-    using Src = typename View::Source;
+    using SrcView = decltype(View::src);
+    using Pre = decltype(View::pre);
+    using Access = SourceAccess<SrcView>;
+    using Src = typename View::Source; // the pixel that is interpolated: the source view's pixel after Pre
     using Pixel = typename View::Pixel;
     using OutPixel = typename Out::Pixel;
+    // packed pixels read as they are: taps and tile slots come straight from memory as dwords
+    static constexpr bool RAW_SOURCE = std::is_same_v<SrcView, PlainView<Src>> && std::is_same_v<Pre, NoTail>;
     static constexpr int SLOT = dev::slot_dwords<Src>();
     static constexpr int OUT_ROW_BYTES = RESIZE_TILE_W * static_cast<int>(sizeof(OutPixel));
     // packed outputs whose four pixels per thread are not one 16-byte piece go out through LDS as whole 16-byte pieces
@@ -375,12 +481,17 @@ struct ResizeJob {
         return rows * (cols | 1) * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * RESIZE_TILE_W * RESIZE_TILE_H + 256;
     }
 
+    // source pixel (x, y) of the resampled window, after the operations fused before the resize
+    __device__ __attribute__((always_inline)) static inline Src fetch(const View& v, int x, int y) {
+        return dev::apply_tail(v.pre, Access::load_one(v.src, x, y));
+    }
+
     // Four consecutive pixels of row y, taps from the staged tile (STAGED) or straight from memory.
     template <bool STAGED, bool INTERIOR>
     __device__ __attribute__((always_inline)) static inline void pixels(const Prog& prog, const unsigned int* tile, const char* window,
                                                                        int sx_lo, int sy_lo, int stride, int x_first, int y, OutPixel* o) {
         const View& v = prog.view;
-        const PlainView<Src>& s = v.src;
+        const SrcView& s = v.src;
         const int ry = y + v.off_y;
         bool row_inside = INTERIOR || y < v.h;
         if constexpr (View::HAS_ROI && !INTERIOR) row_inside = row_inside && ry >= v.y1 && ry <= v.y2;
@@ -412,13 +523,18 @@ struct ResizeJob {
                     b = dev::slot_to_pixel<Src>(sb);
                     c = dev::slot_to_pixel<Src>(sc);
                     d = dev::slot_to_pixel<Src>(sd);
-                } else {
+                } else if constexpr (RAW_SOURCE) {
                     const char* const r0 = window + static_cast<size_t>(t.y1) * s.pitch;
                     const char* const r1 = window + static_cast<size_t>(t.y2r) * s.pitch;
                     a = reinterpret_cast<const Src*>(r0)[t.x1];
                     b = reinterpret_cast<const Src*>(r0)[t.x2r];
                     c = reinterpret_cast<const Src*>(r1)[t.x1];
                     d = reinterpret_cast<const Src*>(r1)[t.x2r];
+                } else {
+                    a = fetch(v, t.x1, t.y1);
+                    b = fetch(v, t.x2r, t.y1);
+                    c = fetch(v, t.x1, t.y2r);
+                    d = fetch(v, t.x2r, t.y2r);
                 }
                 value = fk::detail::bilinear_blend(a, b, c, d, t);
             }
@@ -429,7 +545,7 @@ struct ResizeJob {
     __device__ __attribute__((always_inline)) static inline void run(const ResizeJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char* lds_raw) {
         const Prog& prog = job.plane[N == 1 ? 0u : bz];
         const View& v = prog.view;
-        const PlainView<Src>& s = v.src;
+        const SrcView& s = v.src;
         const int tx0 = static_cast<int>(bx) * RESIZE_TILE_W;
         const int ty0 = static_cast<int>(by) * RESIZE_TILE_H;
         if (tx0 >= v.w || ty0 >= v.h) return; // block outside this plane's own extent
@@ -452,8 +568,9 @@ struct ResizeJob {
         bool staged = false;
         int sx_lo = 0, sy_lo = 0;
         int stride = 0; // slots per tile row
+        // window pixel (0, 0) and the byte range of a window row that belongs to the parent image (raw sources only)
         const char* const window = reinterpret_cast<const char*>(s.data) + static_cast<size_t>(s.oy) * s.pitch +
-                                   static_cast<size_t>(s.ox) * sizeof(Src); // window pixel (0, 0)
+                                   static_cast<size_t>(s.ox) * sizeof(Src);
         const int valid_lo = -s.ox * static_cast<int>(sizeof(Src));
         const int valid_hi = (s.img_w - s.ox) * static_cast<int>(sizeof(Src));
         if (resamples) {
@@ -474,7 +591,15 @@ struct ResizeJob {
                     const char* const row = window + static_cast<size_t>(sy) * s.pitch;
                     for (int c = lane; c < cols; c += 64) {
                         const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
-                        const dev::PixelSlot<Src> px = dev::load_pixel_slot<Src>(row, sx * static_cast<int>(sizeof(Src)), valid_lo, valid_hi);
+                        dev::PixelSlot<Src> px;
+                        if constexpr (RAW_SOURCE) {
+                            px = dev::load_pixel_slot<Src>(row, sx * static_cast<int>(sizeof(Src)), valid_lo, valid_hi);
+                        } else {
+                            const Src value = fetch(v, sx, sy);
+#pragma unroll
+                            for (int i = 0; i < SLOT; ++i) px.w[i] = 0u;
+                            __builtin_memcpy(px.w, &value, sizeof(Src));
+                        }
 #pragma unroll
                         for (int i = 0; i < SLOT; ++i) tile[(r * stride + c) * SLOT + i] = px.w[i];
                     }

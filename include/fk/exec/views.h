@@ -2,8 +2,12 @@
 // ("views") that the hand-written kernels index directly.
 //
 //   PlainView   out(x, y) = img(x + ox, y + oy)                      PerThreadRead<_2D>, possibly under Crop
-//   ResizeView  out(x, y) = bilinear(window, (x + off - roi) * f)     Resize<INTER_LINEAR> over a PlainView, possibly
-//                                                                    under an outer Crop (reads pulled back through it)
+//   YuvView     out(x, y) = {Y, U, V} of pixel (x + ox, y + oy)       ReadYUV<PF>, possibly under Crop
+//   ResizeView  out(x, y) = bilinear(pre(window), (x + off - roi) * f)  Resize<INTER_LINEAR> over one of the above,
+//                                                                    optionally with compute operations fused between
+//                                                                    the read and the resize (`pre`, applied to every
+//                                                                    source pixel), possibly under an outer Crop
+//                                                                    (reads pulled back through it)
 // Folding Crop into an origin is what Crop::exec does one element at a time (reference
 // algorithms/image_processing/crop.h:35-38); the Resize parameters are the ones Resize::build computed
 // (resize.h:105-166).  Chains that do not match keep their generic per-element form.
@@ -11,6 +15,7 @@
 #define FK_EXEC_VIEWS_H
 
 #include "fk/ops/image_processing.h"
+#include "fk/ops/yuv.h"
 
 namespace fk {
 namespace exec {
@@ -27,21 +32,39 @@ struct PlainView {
     int w, h;   // window size: the extent this plane produces
 };
 
-template <typename T, AspectRatio AR>
+// A window of a raw YUV image, seen as {Y, U, V} pixels of the format's base type.
+template <PixelFormat PF>
+struct YuvView {
+    using Base = ColorDepthPixelBaseType<PixelFormatTraits<PF>::depth>;
+    using Pixel = VectorType_t<Base, 3>;
+    using Source = Pixel;
+    static constexpr bool IS_RESIZE = false;
+    static constexpr PixelFormat FORMAT = PF;
+    const Base* data; // first luma (or packed) row of the parent image
+    uint pitch;       // bytes between rows, of every plane
+    int img_w, img_h; // parent image size in pixels; semi-planar chroma rows follow row img_h - 1
+    int ox, oy;       // window origin in the parent
+    int w, h;         // window size: the extent this plane produces
+};
+
+struct NoTail {};
+
+// SrcView: the window that is resampled (its w, h are the clamp limits); Pre: compute operations applied to each of
+// its pixels before interpolation (NoTail for none); T: the pixel type that comes out of Pre.
+template <typename SrcView, typename Pre, typename T, AspectRatio AR>
 struct ResizeView {
     using Source = T;
     using Pixel = VectorType_t<float, cn<T>>;
     static constexpr bool IS_RESIZE = true;
     static constexpr bool HAS_ROI = AR != AspectRatio::IGNORE_AR;
-    PlainView<T> src; // the window that is resampled; its w, h are the clamp limits
+    SrcView src;
+    Pre pre;
     float fx, fy;
     int off_x, off_y;   // added to the output coordinate before resampling (an outer Crop)
     int x1, y1, x2, y2; // destination region that holds the image; the rest is background
     Pixel background;
     int w, h; // the extent this plane produces
 };
-
-struct NoTail {};
 
 template <typename View, typename Tail>
 struct PlaneProgram {
@@ -66,6 +89,17 @@ struct ViewOf<Read<PerThreadRead<ND::_2D, T>>> {
     }
 };
 
+template <PixelFormat PF>
+struct ViewOf<Read<ReadYUV<PF>>> {
+    static constexpr bool supported = true;
+    using type = YuvView<PF>;
+    static type make(const Read<ReadYUV<PF>>& iOp) {
+        const RawImage<PF>& raw = iOp.params;
+        return type{ raw.data.data, raw.data.dims.pitch, static_cast<int>(raw.width), static_cast<int>(raw.height), 0, 0,
+                     static_cast<int>(raw.width), static_cast<int>(raw.height) };
+    }
+};
+
 template <typename Back>
 struct ViewOf<ReadBack<Crop<Back>>, std::enable_if_t<ViewOf<Back>::supported>> {
     static constexpr bool supported = true;
@@ -86,21 +120,61 @@ struct ViewOf<ReadBack<Crop<Back>>, std::enable_if_t<ViewOf<Back>::supported>> {
     }
 };
 
-namespace detail {
-template <typename Back, typename = void>
-struct BackIsPlain : std::false_type {};
+// What a resize resamples: a window view plus the compute operations fused between the read and the resize.
+template <typename IOp, typename = void>
+struct SourceOf {
+    static constexpr bool supported = false;
+};
+template <typename IOp>
+struct SourceOf<IOp, std::enable_if_t<ViewOf<IOp>::supported && !ViewOf<IOp>::type::IS_RESIZE>> {
+    static constexpr bool supported = true;
+    using View = typename ViewOf<IOp>::type;
+    using Pre = NoTail;
+    using Pixel = typename View::Pixel;
+    static View view(const IOp& iOp) { return ViewOf<IOp>::make(iOp); }
+    static Pre pre(const IOp&) { return Pre{}; }
+};
+template <typename Head, typename... ComputeOps>
+struct SourceOf<Read<FusedOperation<Head, ComputeOps...>>,
+                std::enable_if_t<isAnyReadType<Head> && ViewOf<Instantiable<Head>>::supported && !ViewOf<Instantiable<Head>>::type::IS_RESIZE &&
+                                 (sizeof...(ComputeOps) > 0)>> {
+    static constexpr bool supported = true;
+    using IOp = Read<FusedOperation<Head, ComputeOps...>>;
+    using View = typename ViewOf<Instantiable<Head>>::type;
+    using Pre = OperationTuple<ComputeOps...>;
+    using Pixel = typename IOp::Operation::OutputType;
+    static View view(const IOp& iOp) { return ViewOf<Instantiable<Head>>::make(toIOp<Head>(iOp.params.instance)); }
+    static Pre pre(const IOp& iOp) { return fk::detail::tuple_tail(iOp.params); }
+};
+// a crop of a read that is fused with compute operations: the operations commute with the window
 template <typename Back>
-struct BackIsPlain<Back, std::enable_if_t<ViewOf<Back>::supported && !ViewOf<Back>::type::IS_RESIZE>> : std::true_type {};
-} // namespace detail
+struct SourceOf<ReadBack<Crop<Back>>, std::enable_if_t<!ViewOf<Back>::supported && SourceOf<Back>::supported>> {
+    static constexpr bool supported = true;
+    using View = typename SourceOf<Back>::View;
+    using Pre = typename SourceOf<Back>::Pre;
+    using Pixel = typename SourceOf<Back>::Pixel;
+    static View view(const ReadBack<Crop<Back>>& iOp) {
+        View v = SourceOf<Back>::view(iOp.backIOp);
+        const Rect& r = iOp.params;
+        v.ox += static_cast<int>(r.x);
+        v.oy += static_cast<int>(r.y);
+        v.w = r.width;
+        v.h = r.height;
+        return v;
+    }
+    static Pre pre(const ReadBack<Crop<Back>>& iOp) { return SourceOf<Back>::pre(iOp.backIOp); }
+};
 
 template <AspectRatio AR, typename Back>
-struct ViewOf<ReadBack<Resize<InterpolationType::INTER_LINEAR, AR, Back>>, std::enable_if_t<detail::BackIsPlain<Back>::value>> {
+struct ViewOf<ReadBack<Resize<InterpolationType::INTER_LINEAR, AR, Back>>, std::enable_if_t<SourceOf<Back>::supported>> {
     static constexpr bool supported = true;
-    using Source = typename ViewOf<Back>::type::Source;
-    using type = ResizeView<Source, AR>;
+    using Src = SourceOf<Back>;
+    using Source = typename Src::Pixel;
+    using type = ResizeView<typename Src::View, typename Src::Pre, Source, AR>;
     static type make(const ReadBack<Resize<InterpolationType::INTER_LINEAR, AR, Back>>& iOp) {
         type v{};
-        v.src = ViewOf<Back>::make(iOp.backIOp);
+        v.src = Src::view(iOp.backIOp);
+        v.pre = Src::pre(iOp.backIOp);
         const auto& p = iOp.params;
         v.fx = p.src_conv_factors.x;
         v.fy = p.src_conv_factors.y;
