@@ -137,6 +137,43 @@ def other_configs(fk, timer, steps, warmup, only=None):
         ms = time_launches(timer, lambda i: call4(), steps, warmup)
         record("C4_resize_crop_32x128x128", ms, 32 * 128 * 128, 32 * 383 * 383 * 3 + 32 * 128 * 128 * 12)
 
+    # Y1..Y4: the YUV front-end at 4K (raw buffers of random bytes: every value is a legal sample)
+    n4k = 3840 * 2160
+    if want("Y1_nv12_4k_to_rgb_u8c3"):
+        nv12 = rnd_u8(3240, 3840)
+        outs = [torch.empty((2160, 3840, 3), dtype=torch.uint8, device="cuda") for _ in range(3)]
+        calls = [fk.yuv_to_rgb(fk.NV12, fk.RANGE_FULL, fk.BT709, nv12, o, defer=True) for o in outs]
+        ms = time_launches(timer, lambda i: calls[i % 3](), steps, warmup)
+        record("Y1_nv12_4k_to_rgb_u8c3", ms, n4k, n4k * 3 // 2 + n4k * 3)
+        del outs, calls
+    if want("Y2_p010_4k_to_rgba_u16c4"):
+        p010 = torch.randint(-32768, 32767, (3240, 3840), dtype=torch.int16, device="cuda", generator=g)
+        outs = [torch.empty((2160, 3840, 4), dtype=torch.int16, device="cuda") for _ in range(3)]
+        calls = [fk.yuv_to_rgb(fk.P010, fk.RANGE_FULL, fk.BT2020, p010, o, defer=True) for o in outs]
+        ms = time_launches(timer, lambda i: calls[i % 3](), steps, warmup)
+        record("Y2_p010_4k_to_rgba_u16c4", ms, n4k, n4k * 3 + n4k * 8)
+        del outs, calls, p010
+    if want("Y3_uyvy_4k_to_rgb_f32c3"):
+        uyvy = rnd_u8(2160, 7680)
+        outs = [torch.empty((2160, 3840, 3), device="cuda") for _ in range(3)]
+        calls = [fk.yuv_to_rgb(fk.UYVY, fk.RANGE_FULL, fk.BT601, uyvy, o, defer=True) for o in outs]
+        ms = time_launches(timer, lambda i: calls[i % 3](), steps, warmup)
+        record("Y3_uyvy_4k_to_rgb_f32c3", ms, n4k, n4k * 2 + n4k * 12)
+        del outs, calls, uyvy
+    if want("Y4_nv12_crop1920x1080_to_1280x720_split"):
+        nv12 = rnd_u8(3240, 3840)
+        out_y4 = torch.empty((3, 720, 1280), device="cuda")
+        call_y4 = fk.yuv_crop_resize_norm_split(fk.NV12, fk.RANGE_FULL, fk.BT709, nv12, (3840, 2160), (960, 540, 1920, 1080), out_y4, 255.0, defer=True)
+        ms = time_launches(timer, lambda i: call_y4(), steps, warmup)
+        record("Y4_nv12_crop1920x1080_to_1280x720_split", ms, 1280 * 720, 1920 * 1080 * 3 // 2 + 1280 * 720 * 12,
+               "the README's backwards-vertical-fusion example: only the crop's YUV samples are read")
+    if want("Y5_nv12_crop640x360_to_1920x1080_split"):
+        nv12 = rnd_u8(3240, 3840)
+        out_y5 = torch.empty((3, 1080, 1920), device="cuda")
+        call_y5 = fk.yuv_crop_resize_norm_split(fk.NV12, fk.RANGE_FULL, fk.BT709, nv12, (3840, 2160), (1600, 900, 640, 360), out_y5, 255.0, defer=True)
+        ms = time_launches(timer, lambda i: call_y5(), steps, warmup)
+        record("Y5_nv12_crop640x360_to_1920x1080_split", ms, 1920 * 1080, 640 * 360 * 3 // 2 + 1920 * 1080 * 12)
+
     # C5: four chains over one 8192x8192 uchar4 image in one launch
     if not want("C5_divergent4_8192x8192"):
         return res

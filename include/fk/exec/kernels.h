@@ -129,12 +129,49 @@ __device__ __attribute__((always_inline)) inline void store_one(const SplitOut<O
     if constexpr (cn<O> == 4) reinterpret_cast<B*>(row + 3 * out.chan_stride)[x] = v.w;
 }
 
+// N elements of a 1- or 2-byte type into whole dwords, in registers (a byte-wise copy would go through scratch memory)
+template <int N, typename B>
+__device__ __attribute__((always_inline)) inline void pack_elements(const B* e, unsigned int* w) {
+    if constexpr (sizeof(B) >= 4) {
+        __builtin_memcpy(w, e, N * sizeof(B));
+    } else {
+        constexpr int PER = 4 / static_cast<int>(sizeof(B));
+        static_assert(N % PER == 0, "whole dwords");
+#pragma unroll
+        for (int i = 0; i < N / PER; ++i) {
+            unsigned int word = 0u;
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                using U = std::make_unsigned_t<std::conditional_t<std::is_same_v<B, bool>, unsigned char, B>>;
+                word |= static_cast<unsigned int>(static_cast<U>(e[i * PER + j])) << (8 * static_cast<int>(sizeof(B)) * j);
+            }
+            w[i] = word;
+        }
+    }
+}
+// K pixels as the dwords they occupy in memory
+template <int K, typename O>
+__device__ __attribute__((always_inline)) inline void pack_pixels(const O* v, unsigned int* w) {
+    if constexpr (sizeof(O) % 4 == 0) {
+        __builtin_memcpy(w, v, K * sizeof(O));
+    } else {
+        using B = VBase<O>;
+        B e[K * cn<O>];
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+#pragma unroll
+            for (int c = 0; c < cn<O>; ++c) e[k * cn<O> + c] = vectorAt(c, v[k]);
+        }
+        pack_elements<K * cn<O>>(e, w);
+    }
+}
+
 // K consecutive pixels starting at x0 (caller guarantees the alignment that chunk_bytes asks for)
 template <int K, bool STREAM = false, typename O>
 __device__ __attribute__((always_inline)) inline void store_group(const PackedOut<O>& out, int x0, int y, int z, const O* v) {
     constexpr int NB = K * static_cast<int>(sizeof(O));
     unsigned int w[NB / 4];
-    __builtin_memcpy(w, v, NB);
+    pack_pixels<K>(v, w);
     char* const row = reinterpret_cast<char*>(out.data) + static_cast<size_t>(z) * out.z_stride + static_cast<size_t>(y) * out.pitch;
     // a thread's K pixels are one transaction only when they fill exactly one piece
     store_words<NB, STREAM && NB == chunk_bytes(NB)>(row + static_cast<size_t>(x0) * sizeof(O), w);
@@ -150,7 +187,7 @@ __device__ __attribute__((always_inline)) inline void store_group(const SplitOut
 #pragma unroll
         for (int k = 0; k < K; ++k) ch[k] = vectorAt(c, v[k]);
         unsigned int w[NB / 4];
-        __builtin_memcpy(w, ch, NB);
+        pack_elements<K>(ch, w);
         store_words<NB, STREAM && NB == chunk_bytes(NB)>(row + c * out.chan_stride + static_cast<size_t>(x0) * sizeof(B), w);
     }
 }
@@ -294,6 +331,71 @@ struct PointwiseJob {
     unsigned grid_x, grid_y;
     size_t lds_bytes() const { return LDS_BYTES; }
 
+    // A block that lies on one row and owns `span` pixels of it from pixel bx0 on (a whole number of thread groups, so
+    // the span is whole 16-byte pieces on both sides).  FULL: span is the block's whole 256*K pixels, nothing is guarded.
+    template <bool FULL>
+    __device__ __attribute__((always_inline)) static inline void row_block(const PointwiseJob& job, const Plane& pl, int bx0, int span, int x0, int y,
+                                                                          unsigned bz, int tid, unsigned char* lds) {
+        const View& v = pl.prog.view;
+        dev::u32x4* const stage = reinterpret_cast<dev::u32x4*>(lds);
+        const bool active = FULL || x0 < v.w;
+        Src in[K];
+        if constexpr (STAGE_IN) {
+            const dev::u32x4* const g = reinterpret_cast<const dev::u32x4*>(Access::row(v, y) + static_cast<size_t>(bx0) * sizeof(Src));
+            const int pieces = span * static_cast<int>(sizeof(Src)) / 16;
+#pragma unroll
+            for (int j = 0; j < IN_BYTES / 16; ++j) {
+                if (FULL || j * BLOCK_THREADS + tid < pieces) stage[j * BLOCK_THREADS + tid] = g[j * BLOCK_THREADS + tid];
+            }
+            dev::block_sync();
+            if (active) {
+                dev::u32x4 mine[IN_BYTES / 16];
+#pragma unroll
+                for (int j = 0; j < IN_BYTES / 16; ++j) mine[j] = stage[tid * (IN_BYTES / 16) + j];
+                __builtin_memcpy(in, mine, IN_BYTES);
+            }
+        } else {
+            if (active) Access::template load_group<K>(v, x0, y, in);
+        }
+        OutPixel o[K];
+        if (active) {
+#pragma unroll
+            for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
+        }
+        if constexpr (STAGE_OUT) {
+            if constexpr (STAGE_IN) dev::block_sync(); // every thread has taken its input out of the buffer
+            if (active) {
+                unsigned int w[OUT_BYTES / 4];
+                dev::pack_pixels<K>(o, w);
+#pragma unroll
+                for (int j = 0; j < OUT_BYTES / 16; ++j) {
+                    dev::u32x4 piece;
+                    piece.x = w[4 * j]; piece.y = w[4 * j + 1]; piece.z = w[4 * j + 2]; piece.w = w[4 * j + 3];
+                    stage[tid * (OUT_BYTES / 16) + j] = piece;
+                }
+            }
+            dev::block_sync();
+            dev::u32x4* const g = reinterpret_cast<dev::u32x4*>(
+                reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
+                static_cast<size_t>(y) * job.out.pitch + static_cast<size_t>(bx0) * sizeof(OutPixel));
+            const int pieces = span * static_cast<int>(sizeof(OutPixel)) / 16;
+            if ((pl.flags & FLAG_STREAM_STORES) != 0u) {
+#pragma unroll
+                for (int j = 0; j < OUT_BYTES / 16; ++j) {
+                    if (FULL || j * BLOCK_THREADS + tid < pieces) dev::store_piece<true>(g + j * BLOCK_THREADS + tid, stage[j * BLOCK_THREADS + tid]);
+                }
+            } else {
+#pragma unroll
+                for (int j = 0; j < OUT_BYTES / 16; ++j) {
+                    if (FULL || j * BLOCK_THREADS + tid < pieces) g[j * BLOCK_THREADS + tid] = stage[j * BLOCK_THREADS + tid];
+                }
+            }
+        } else if (active) {
+            if ((pl.flags & FLAG_STREAM_STORES) != 0u) dev::store_group<K, true>(job.out, x0, y, static_cast<int>(bz), o);
+            else dev::store_group<K>(job.out, x0, y, static_cast<int>(bz), o);
+        }
+    }
+
     __device__ __attribute__((always_inline)) static inline void run(const PointwiseJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char* lds) {
         const Plane& pl = job.plane[N == 1 ? 0u : bz];
         const View& v = pl.prog.view;
@@ -303,65 +405,12 @@ struct PointwiseJob {
         const int y = static_cast<int>(by) * (BLOCK_THREADS >> job.tx_shift) + (tid >> job.tx_shift);
 
         if constexpr (STAGE_IN || STAGE_OUT) {
-            // block-uniform: the whole block lies on one row; `span` pixels of that row are the block's, a whole number
-            // of thread groups, so the span is whole 16-byte pieces on both sides
+            // block-uniform decisions
             const int bx0 = static_cast<int>(bx) * BLOCK_THREADS * K; // first pixel of the block
             const int span = v.w - bx0 < BLOCK_THREADS * K ? v.w - bx0 : BLOCK_THREADS * K;
-            const bool rowwise = (pl.flags & FLAG_VECTOR_IO) != 0u && job.tx_shift == 8u && y < v.h && span > 0 && span % K == 0;
-            if (rowwise) {
-                dev::u32x4* const stage = reinterpret_cast<dev::u32x4*>(lds);
-                const bool active = x0 < v.w;
-                Src in[K];
-                if constexpr (STAGE_IN) {
-                    const dev::u32x4* const g = reinterpret_cast<const dev::u32x4*>(Access::row(v, y) + static_cast<size_t>(bx0) * sizeof(Src));
-                    const int pieces = span * static_cast<int>(sizeof(Src)) / 16;
-#pragma unroll
-                    for (int j = 0; j < IN_BYTES / 16; ++j) {
-                        if (j * BLOCK_THREADS + tid < pieces) stage[j * BLOCK_THREADS + tid] = g[j * BLOCK_THREADS + tid];
-                    }
-                    dev::block_sync();
-                    if (active) {
-                        dev::u32x4 mine[IN_BYTES / 16];
-#pragma unroll
-                        for (int j = 0; j < IN_BYTES / 16; ++j) mine[j] = stage[tid * (IN_BYTES / 16) + j];
-                        __builtin_memcpy(in, mine, IN_BYTES);
-                    }
-                } else {
-                    if (active) Access::template load_group<K>(v, x0, y, in);
-                }
-                OutPixel o[K];
-                if (active) {
-#pragma unroll
-                    for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
-                }
-                if constexpr (STAGE_OUT) {
-                    if constexpr (STAGE_IN) dev::block_sync(); // every thread has taken its input out of the buffer
-                    if (active) {
-                        dev::u32x4 mine[OUT_BYTES / 16];
-                        __builtin_memcpy(mine, o, OUT_BYTES);
-#pragma unroll
-                        for (int j = 0; j < OUT_BYTES / 16; ++j) stage[tid * (OUT_BYTES / 16) + j] = mine[j];
-                    }
-                    dev::block_sync();
-                    dev::u32x4* const g = reinterpret_cast<dev::u32x4*>(
-                        reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
-                        static_cast<size_t>(y) * job.out.pitch + static_cast<size_t>(bx0) * sizeof(OutPixel));
-                    const int pieces = span * static_cast<int>(sizeof(OutPixel)) / 16;
-                    if ((pl.flags & FLAG_STREAM_STORES) != 0u) {
-#pragma unroll
-                        for (int j = 0; j < OUT_BYTES / 16; ++j) {
-                            if (j * BLOCK_THREADS + tid < pieces) dev::store_piece<true>(g + j * BLOCK_THREADS + tid, stage[j * BLOCK_THREADS + tid]);
-                        }
-                    } else {
-#pragma unroll
-                        for (int j = 0; j < OUT_BYTES / 16; ++j) {
-                            if (j * BLOCK_THREADS + tid < pieces) g[j * BLOCK_THREADS + tid] = stage[j * BLOCK_THREADS + tid];
-                        }
-                    }
-                } else if (active) {
-                    if ((pl.flags & FLAG_STREAM_STORES) != 0u) dev::store_group<K, true>(job.out, x0, y, static_cast<int>(bz), o);
-                    else dev::store_group<K>(job.out, x0, y, static_cast<int>(bz), o);
-                }
+            if ((pl.flags & FLAG_VECTOR_IO) != 0u && job.tx_shift == 8u && y < v.h && span > 0 && span % K == 0) {
+                if (span == BLOCK_THREADS * K) row_block<true>(job, pl, bx0, span, x0, y, bz, tid, lds);
+                else row_block<false>(job, pl, bx0, span, x0, y, bz, tid, lds);
                 return;
             }
         }

@@ -107,12 +107,26 @@ public:
     FK_HD_STATIC OutputType exec(const InputType& input) {
         constexpr O hi = maxValue<O>;
         constexpr O lo = minValue<O>;
-        if (cxp::cmp_greater(input, hi)) return hi;
-        if (cxp::cmp_less(input, lo)) return lo;
-        if constexpr (std::is_floating_point_v<I> && std::is_integral_v<O>) {
-            return static_cast<O>(cxp::round(input));
+        if constexpr (std::is_floating_point_v<I> && std::is_integral_v<O> && sizeof(O) < sizeof(int)) {
+            // The same value as the general form below for every finite input, written without branches: clamp first
+            // (the limits are integers, so rounding leaves them alone), then round half away from zero through int.
+            const I above = static_cast<I>(hi), below = static_cast<I>(lo);
+            I clamped{};
+            if constexpr (std::is_same_v<I, float>) clamped = __builtin_fmaxf(__builtin_fminf(input, above), below);
+            else clamped = static_cast<I>(__builtin_fmax(__builtin_fmin(static_cast<double>(input), static_cast<double>(above)), static_cast<double>(below)));
+            if constexpr (std::is_unsigned_v<O>) {
+                return static_cast<O>(static_cast<int>(clamped + I(0.5))); // clamped >= 0, and (int)(0 - 0.5) == (int)(0 + 0.5)
+            } else {
+                return static_cast<O>(static_cast<int>(clamped + (clamped > I(0) ? I(0.5) : I(-0.5))));
+            }
         } else {
-            return static_cast<O>(input);
+            if (cxp::cmp_greater(input, hi)) return hi;
+            if (cxp::cmp_less(input, lo)) return lo;
+            if constexpr (std::is_floating_point_v<I> && std::is_integral_v<O>) {
+                return static_cast<O>(cxp::round(input));
+            } else {
+                return static_cast<O>(input);
+            }
         }
     }
 };
