@@ -55,7 +55,11 @@ CAPI_SIGNATURES = {
     "fk_write_yuv": [_i, _vp, _sz, _i, _i, _vp, _sz, _vp],
     "fk_yuv_to_rgb": [_i, _i, _i, _i, _i, _vp, _sz, _i, _i, _vp, _sz, _vp],
     "fk_yuv_crop_resize_norm_split": [_i, _i, _i, _vp, _sz, _i, _i, Rect, _i, _i, _f, _vp, _vp],
+    "fk_border_crop_u8c3": [_i, _vp, _i, _i, _sz, _i, _i, _i, _i, C.POINTER(C.c_uint8), _vp, _sz, _vp],
+    "fk_warp_u8c3_f32c3": [_i, C.POINTER(C.c_float), _vp, _i, _i, _sz, _i, _i, _vp, _sz, _vp],
 }
+BORDER_CONSTANT, BORDER_REPLICATE, BORDER_REFLECT, BORDER_WRAP, BORDER_REFLECT_101 = 0, 1, 2, 3, 4
+WARP_AFFINE, WARP_PERSPECTIVE = 0, 1
 # PixelFormat / ColorRange / ColorPrimitives values of include/fk_capi.h
 NV12, NV21, P010, P210, Y210, UYVY = 0, 1, 3, 6, 8, 10
 RANGE_LIMITED, RANGE_FULL = 0, 1
@@ -334,4 +338,30 @@ def yuv_crop_resize_norm_split(fmt, color_range, primaries, raw, size, crop, out
     assert out.is_contiguous()
     _deferred = _call(capi.fk_yuv_crop_resize_norm_split, (fmt, color_range, primaries, p, pitch, size[0], size[1], Rect(*[int(v) for v in crop]),
                                                            dw, dh, float(div_v), C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+# ---- BorderReader and Warping ------------------------------------------------------------------------------------------
+
+def border_crop_u8c3(border_type, src, left, top, out, value=(0, 0, 0), stream=None, defer=False):
+    """src: (h, w, 3) uint8 seen through BorderReader<border_type>; out: (dst_h, dst_w, 3) uint8 = the window whose origin
+    is (-left, -top) in image coordinates."""
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    q, dw, dh, out_pitch = _image(out, "uint8")
+    val = (C.c_uint8 * 3)(*[int(v) for v in value])
+    _deferred = _call(capi.fk_border_crop_u8c3, (border_type, p, w, h, pitch, int(left), int(top), dw, dh, val, q, out_pitch, _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def warp_u8c3_f32c3(warp_type, matrix, src, out, stream=None, defer=False):
+    """matrix: 6 (affine) or 9 (perspective) floats, row-major, destination -> source; out: (dst_h, dst_w, 3) float32."""
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    q, dw, dh, out_pitch = _image(out, "float32")
+    flat = [float(v) for row in matrix for v in (row if hasattr(row, "__len__") else [row])]
+    if len(flat) != (6 if warp_type == WARP_AFFINE else 9):
+        raise FkError("matrix must be 2x3 (affine) or 3x3 (perspective)")
+    m = (C.c_float * len(flat))(*flat)
+    _deferred = _call(capi.fk_warp_u8c3_f32c3, (warp_type, m, p, w, h, pitch, dw, dh, q, out_pitch, _stream(stream)), defer)
     return _deferred if defer else out

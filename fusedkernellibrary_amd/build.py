@@ -1,7 +1,7 @@
 """Build recipe of the native libraries (hipcc, gfx950 only).
 
   libfk_hip_rt.so   the C runtime ABI of include/fk_hip_rt.h (csrc/fk_hip_rt.cpp)
-  libfk_capi.so     the chain entry points of include/fk_capi.h (csrc/fk_capi.hip, csrc/fk_capi_yuv.hip), i.e. the
+  libfk_capi.so     the chain entry points of include/fk_capi.h (csrc/fk_capi*.hip), i.e. the
                     fused kernels instantiated from the fk:: templates under include/fk/
 
 Run as `python -m fusedkernellibrary_amd.build`; outputs land beside this file.
@@ -43,7 +43,7 @@ def build_runtime():
     return out
 
 
-CAPI_SOURCES = ("fk_capi.hip", "fk_capi_yuv.hip")
+CAPI_SOURCES = ("fk_capi.hip", "fk_capi_yuv.hip", "fk_capi_border_warp.hip")
 
 
 def build_capi(extra_defines=(), name="libfk_capi.so"):

@@ -107,6 +107,46 @@ struct RawPtr {
     enum { ND = static_cast<int>(D) };
 };
 
+// Small fixed-size arrays carried by value inside operation parameters (core/data/rawptr.h:106-184): data[H][W].
+template <int W>
+struct StaticPtrDims1D {
+    static constexpr uint width{ W };
+};
+template <int W, int H>
+struct StaticPtrDims2D {
+    static constexpr uint width{ W };
+    static constexpr uint height{ H };
+};
+template <int W, int H, int P>
+struct StaticPtrDims3D {
+    static constexpr uint width{ W };
+    static constexpr uint height{ H };
+    static constexpr uint planes{ P };
+};
+template <typename Dims, typename T>
+struct StaticRawPtr;
+template <typename T, int W>
+struct StaticRawPtr<StaticPtrDims1D<W>, T> {
+    using type = T;
+    T data[W];
+    static constexpr StaticPtrDims1D<W> dims{};
+    static constexpr ND NDim{ ND::_1D };
+};
+template <typename T, int W, int H>
+struct StaticRawPtr<StaticPtrDims2D<W, H>, T> {
+    using type = T;
+    T data[H][W];
+    static constexpr StaticPtrDims2D<W, H> dims{};
+    static constexpr ND NDim{ ND::_2D };
+};
+template <typename T, int W, int H, int P>
+struct StaticRawPtr<StaticPtrDims3D<W, H, P>, T> {
+    using type = T;
+    T data[P][H][W];
+    static constexpr StaticPtrDims3D<W, H, P> dims{};
+    static constexpr ND NDim{ ND::_3D };
+};
+
 // Byte-pitch addressing of a RawPtr (core/data/rawptr.h:186-239).
 template <ND D>
 struct PtrAccessor;

@@ -5,6 +5,8 @@
 
 #include "fk/exec/executor.h"
 #include "fk/ops/yuv.h"
+#include "fk/ops/border_reader.h"
+#include "fk/ops/warping.h"
 
 namespace fk {
 

@@ -119,6 +119,25 @@ int fk_yuv_to_rgb(int format, int range, int primaries, int alpha, int float_out
 int fk_yuv_crop_resize_norm_split(int format, int range, int primaries, const void* src, size_t src_pitch, int width, int height,
                                   fk_rect crop, int dst_w, int dst_h, float div_v, float* dst, void* stream);
 
+/* ---- BorderReader and Warping ------------------------------------------------------------------------------ */
+
+/* BorderType, algorithms/image_processing/border_reader.h:26-36 (the types implemented there) */
+enum { FK_BORDER_CONSTANT = 0, FK_BORDER_REPLICATE = 1, FK_BORDER_REFLECT = 2, FK_BORDER_WRAP = 3, FK_BORDER_REFLECT_101 = 4 };
+/* WarpType, algorithms/image_processing/warping.h:25 */
+enum { FK_WARP_AFFINE = 0, FK_WARP_PERSPECTIVE = 1 };
+
+/* PerThreadRead<_2D,uchar3> -> BorderReader<border_type>(value) -> Crop(Rect(-left, -top, dst_w, dst_h)) ->
+ * PerThreadWrite<_2D,uchar3> (border_reader.h:141-277, crop.h:35-38): a window of the image extended by its border
+ * rule; with left, top >= 0 and a larger destination this is the image with a border around it.  `value` is used by
+ * FK_BORDER_CONSTANT only. */
+int fk_border_crop_u8c3(int border_type, const void* src, int w, int h, size_t src_pitch, int left, int top, int dst_w, int dst_h,
+                        const uint8_t value[3], void* dst, size_t dst_pitch, void* stream);
+/* PerThreadRead<_2D,uchar3> -> Warping<warp_type>(matrix, dst size) -> PerThreadWrite<_2D,float3> (warping.h:43-108):
+ * matrix is row-major 2x3 (affine) or 3x3 (perspective) and maps destination to source coordinates; destinations whose
+ * source point falls outside the image are zero. */
+int fk_warp_u8c3_f32c3(int warp_type, const float* matrix, const void* src, int w, int h, size_t src_pitch, int dst_w, int dst_h,
+                       void* dst, size_t dst_pitch, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -2,7 +2,7 @@
 
 `oracle()` loads oracle/libfkoracle.so, the plain-C restatement of the reference's CPU executor
 (fk_oracle.c); `reference()` loads oracle/_ref/libfkref.so, the reference's own headers compiled for
-its CPU backend (ref_driver.cpp, plus ref_driver_yuv.cpp in libfkref_yuv.so), or returns None when that build is absent.  Both are built by
+its CPU backend (ref_driver.cpp, plus ref_driver_yuv.cpp and ref_driver_border_warp.cpp in libraries of their own), or returns None when that build is absent.  Both are built by
 oracle/Makefile.  Only tests, the smoke check and the CPU-baseline leg of the benchmark import this
 module; the shipped library never does.
 """
@@ -21,6 +21,9 @@ YUV_FORMATS = {"NV12": NV12, "NV21": NV21, "P010": P010, "P210": P210, "Y210": Y
 RANGE_LIMITED, RANGE_FULL = 0, 1
 BT601, BT709, BT2020 = 0, 1, 2
 # the (range, primaries) pairs for which the reference defines a YCbCr -> RGB matrix
+BORDER_CONSTANT, BORDER_REPLICATE, BORDER_REFLECT, BORDER_WRAP, BORDER_REFLECT_101 = 0, 1, 2, 3, 4
+BORDER_TYPES = {"CONSTANT": 0, "REPLICATE": 1, "REFLECT": 2, "WRAP": 3, "REFLECT_101": 4}
+WARP_AFFINE, WARP_PERSPECTIVE = 0, 1
 YUV_MATRICES = [(RANGE_FULL, BT601), (RANGE_FULL, BT709), (RANGE_LIMITED, BT709), (RANGE_FULL, BT2020)]
 
 
@@ -82,11 +85,22 @@ def build(with_reference=True):
 class _Lib:
     """Thin numpy-facing wrapper; `ref=True` talks to the reference driver (literal host semantics)."""
 
-    def __init__(self, cdll, ref, yuv_cdll=None):
+    def __init__(self, cdll, ref, yuv_cdll=None, bw_cdll=None):
         self.c = cdll
         self.ref = ref
         self.yuv = yuv_cdll
+        self.bw = bw_cdll
         pre = "fkr_" if ref else "fko_"
+        if bw_cdll is not None:
+            _v = C.c_void_p
+            fn = getattr(bw_cdll, pre + "border_crop_u8c3")
+            fn.argtypes, fn.restype = [_i, _v, _i, _i, _sz, _i, _i, _i, _i, _v, _v, _sz], C.c_int
+            fn = getattr(bw_cdll, pre + "warp_coords")
+            fn.argtypes, fn.restype = [_i, _v, _i, _i, _v], None
+            fn = getattr(bw_cdll, pre + "warp_u8c3_f32c3")
+            fn.argtypes, fn.restype = [_i, _v, _v, _i, _i, _sz, _i, _i] + ([] if ref else [_i]) + [_v, _sz], C.c_int
+            if not ref:
+                bw_cdll.fko_border_index.argtypes, bw_cdll.fko_border_index.restype = [_i, _i, _i], C.c_int
         if yuv_cdll is not None:
             _v = C.c_void_p
             for name, sig in {"read_yuv": [_i, _v, _sz, _i, _i, _v, _sz], "write_yuv": [_i, _v, _sz, _i, _i, _v, _sz],
@@ -294,6 +308,42 @@ class _Lib:
         return out
 
 
+    # ---- BorderReader and Warping ----
+    def _bw_fn(self, name):
+        if self.bw is None:
+            raise RuntimeError("the border / warp checker library is not built")
+        return getattr(self.bw, ("fkr_" if self.ref else "fko_") + name)
+
+    def border_index(self, border_type, i, n):
+        return int(self.bw.fko_border_index(border_type, i, n))
+
+    def border_crop_u8c3(self, border_type, src, left, top, dst, value=(0, 0, 0)):
+        """src (h, w, 3) uint8 seen through BorderReader<type>, window of dst = (w, h) pixels whose origin is (-left, -top)."""
+        h, w, _ = src.shape
+        out = np.empty((dst[1], dst[0], 3), np.uint8)
+        val = np.array(value, np.uint8)
+        self._check(self._bw_fn("border_crop_u8c3")(border_type, _p(src), w, h, src.strides[0], left, top, dst[0], dst[1], _p(val),
+                                                     _p(out), out.strides[0]))
+        return out
+
+    def warp_coords(self, warp_type, matrix, x, y):
+        m = np.ascontiguousarray(matrix, np.float32).ravel()
+        out = np.empty(2, np.float32)
+        self._bw_fn("warp_coords")(warp_type, _p(m), x, y, _p(out))
+        return out
+
+    def warp_u8c3_f32c3(self, warp_type, matrix, src, dst, quirk=0):
+        """matrix: 2x3 (affine) or 3x3 (perspective), destination -> source coordinates."""
+        h, w, _ = src.shape
+        m = np.ascontiguousarray(matrix, np.float32).ravel()
+        out = np.empty((dst[1], dst[0], 3), np.float32)
+        args = [warp_type, _p(m), _p(src), w, h, src.strides[0], dst[0], dst[1]]
+        if not self.ref:
+            args.append(quirk)
+        self._check(self._bw_fn("warp_u8c3_f32c3")(*args, _p(out), out.strides[0]))
+        return out
+
+
 _cache = {}
 
 
@@ -303,7 +353,7 @@ def oracle():
         if not os.path.exists(path):
             build(with_reference=False)
         cdll = C.CDLL(path)
-        _cache["o"] = _Lib(cdll, ref=False, yuv_cdll=cdll)
+        _cache["o"] = _Lib(cdll, ref=False, yuv_cdll=cdll, bw_cdll=cdll)
     return _cache["o"]
 
 
@@ -313,5 +363,7 @@ def reference():
         path = os.path.join(_HERE, "_ref", "libfkref.so")
         yuv_path = os.path.join(_HERE, "_ref", "libfkref_yuv.so")
         yuv = C.CDLL(yuv_path) if os.path.exists(yuv_path) else None
-        _cache["r"] = _Lib(C.CDLL(path), ref=True, yuv_cdll=yuv) if os.path.exists(path) else None
+        bw_path = os.path.join(_HERE, "_ref", "libfkref_border_warp.so")
+        bw = C.CDLL(bw_path) if os.path.exists(bw_path) else None
+        _cache["r"] = _Lib(C.CDLL(path), ref=True, yuv_cdll=yuv, bw_cdll=bw) if os.path.exists(path) else None
     return _cache["r"]

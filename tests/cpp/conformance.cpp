@@ -132,6 +132,21 @@ static_assert(NormalizeColorRangeDepth<float3, ColorDepth::p8bit>::exec(float3{ 
               SaturateDenormalizePixel<float3, uchar3, ColorDepth::p8bit>::exec(float3{ -0.5f, 0.5f, 1.5f }).y == 127 &&
               SaturateDenormalizePixel<float3, uchar3, ColorDepth::p8bit>::exec(float3{ -0.5f, 0.5f, 1.5f }).z == 255);
 
+// BorderReader and Warping builders (tests/algorithm/test_border_reader.h:21-30, test_warp.h:20-32 of the reference)
+constexpr auto kBorder = BorderReader<BorderType::CONSTANT>::build(kRead, make_set<uchar3>(0));
+static_assert(std::is_same_v<std::decay_t<decltype(kBorder)>, ReadBack<BorderReader<BorderType::CONSTANT, Read<ReadU3>>>>);
+constexpr auto kWarped = kRead.then(Warping<WarpType::Perspective>::build(WarpingParameters<WarpType::Perspective>{}));
+static_assert(std::is_same_v<std::decay_t<decltype(kWarped)>, ReadBack<Warping<WarpType::Perspective, Read<ReadU3>>>>);
+constexpr auto kPadded = kRead.then(BorderReader<BorderType::REFLECT>::build<uchar3>()).then(Crop<>::build(Rect(static_cast<uint>(-4), static_cast<uint>(-4), 72, 40)));
+static_assert(kPadded.getActiveThreads() == ActiveThreads(72, 40, 1) && std::is_same_v<std::decay_t<decltype(kPadded)>::Operation::OutputType, uchar3>);
+static_assert(kRead.then(BorderReader<BorderType::CONSTANT>::build(uchar3{ 1, 2, 3 })).params.value.z == 3);
+static_assert(detail::border_index<BorderType::REFLECT>(-6, 8) == 5 && detail::border_index<BorderType::REFLECT>(14, 8) == 1 &&
+              detail::border_index<BorderType::REFLECT_101>(-6, 8) == 6 && detail::border_index<BorderType::REFLECT_101>(14, 8) == 0 &&
+              detail::border_index<BorderType::WRAP>(-6, 8) == 2 && detail::border_index<BorderType::WRAP>(14, 8) == 6 &&
+              detail::border_index<BorderType::REPLICATE>(-6, 8) == 0 && detail::border_index<BorderType::REPLICATE>(14, 8) == 7,
+              "the border diagrams of border_reader.h:26-33");
+static_assert(sizeof(WarpingParameters<WarpType::Affine>) == 32 && sizeof(WarpingParameters<WarpType::Perspective>) == 44);
+
 // DPP tags
 static_assert(TransformDPP<>::PAR_ARCH == ParArch::GPU_AMD && defaultParArch == ParArch::GPU_AMD && Stream::parArch() == ParArch::GPU_AMD);
 static_assert(exec::pixels_per_thread<float3, float3, false>() == 4 && exec::pixels_per_thread<uchar4, uchar, false>() == 4 &&
