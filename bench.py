@@ -174,6 +174,29 @@ def other_configs(fk, timer, steps, warmup, only=None):
         ms = time_launches(timer, lambda i: call_y5(), steps, warmup)
         record("Y5_nv12_crop640x360_to_1920x1080_split", ms, 1920 * 1080, 640 * 360 * 3 // 2 + 1920 * 1080 * 12)
 
+    # B1, W1, W2: border and warp chains over the 4K uchar3 frame
+    if want("B1_reflect101_border64_4k_u8c3"):
+        outs = [torch.empty((2160 + 128, 3840 + 128, 3), dtype=torch.uint8, device="cuda") for _ in range(3)]
+        calls = [fk.border_crop_u8c3(fk.BORDER_REFLECT_101, img4k, 64, 64, o, defer=True) for o in outs]
+        ms = time_launches(timer, lambda i: calls[i % 3](), steps, warmup)
+        record("B1_reflect101_border64_4k_u8c3", ms, 3968 * 2288, n4k * 3 + 3968 * 2288 * 3)
+        del outs, calls
+    if want("W1_affine_rot5deg_4k_to_4k_f32c3"):
+        import math
+        c, s_ = math.cos(math.radians(5.0)), math.sin(math.radians(5.0))
+        rot = [[c, -s_, 1920 - c * 1920 + s_ * 1080], [s_, c, 1080 - s_ * 1920 - c * 1080]]  # about the image centre
+        outs = [torch.empty((2160, 3840, 3), device="cuda") for _ in range(3)]
+        calls = [fk.warp_u8c3_f32c3(fk.WARP_AFFINE, rot, img4k, o, defer=True) for o in outs]
+        ms = time_launches(timer, lambda i: calls[i % 3](), steps, warmup)
+        record("W1_affine_rot5deg_4k_to_4k_f32c3", ms, n4k, n4k * 3 + n4k * 12, "source bytes counted once for the whole frame")
+        del outs, calls
+    if want("W2_perspective_4k_to_1920x1080_f32c3"):
+        per = [[2.0, 0.1, 0.0], [0.05, 2.0, 0.0], [2e-5, 1e-5, 1.0]]
+        out_w2 = torch.empty((1080, 1920, 3), device="cuda")
+        call_w2 = fk.warp_u8c3_f32c3(fk.WARP_PERSPECTIVE, per, img4k, out_w2, defer=True)
+        ms = time_launches(timer, lambda i: call_w2(), steps, warmup)
+        record("W2_perspective_4k_to_1920x1080_f32c3", ms, 1920 * 1080, 1920 * 1080 * 4 * 3 + 1920 * 1080 * 12, "four taps per output pixel, 2x down-scaling: no tap is shared")
+
     # C5: four chains over one 8192x8192 uchar4 image in one launch
     if not want("C5_divergent4_8192x8192"):
         return res

@@ -4,6 +4,8 @@
   libfk_capi.so     the chain entry points of include/fk_capi.h (csrc/fk_capi*.hip), i.e. the
                     fused kernels instantiated from the fk:: templates under include/fk/
 
+  benchmarks/reference_sweeps   the reference's benchmark sweeps (benchmarks/reference_sweeps.cpp), a program
+
 Run as `python -m fusedkernellibrary_amd.build`; outputs land beside this file.
 """
 import os
@@ -78,6 +80,14 @@ def build_cpp_tests():
     return outs
 
 
+def build_benchmarks():
+    """benchmarks/reference_sweeps: the reference's four benchmark sweeps as user code of the operator API."""
+    src = os.path.join(HERE, "benchmarks", "reference_sweeps.cpp")
+    out = os.path.join(HERE, "benchmarks", "reference_sweeps")
+    _run([hipcc(), "-x", "hip", src, "-I" + INCLUDE, *DEVICE_FLAGS, "-L" + HERE, "-lfk_hip_rt", "-Wl,-rpath,$ORIGIN/..", "-o", out])
+    return out
+
+
 def build_literal_capi():
     """The same chain entry points built with the reference's host-branch interpolation (bilinear row index taken from
     the x coordinate): only there to show parity with the reference CPU backend's own output where that is defined."""
@@ -88,8 +98,8 @@ def build_all():
     """Everything, the independent hipcc runs side by side (each is single-threaded)."""
     from concurrent.futures import ThreadPoolExecutor
     outs = [build_runtime()]  # the others link against it
-    with ThreadPoolExecutor(max_workers=3) as pool:
-        jobs = [pool.submit(build_capi), pool.submit(build_literal_capi), pool.submit(build_cpp_tests)]
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        jobs = [pool.submit(build_capi), pool.submit(build_literal_capi), pool.submit(build_cpp_tests), pool.submit(build_benchmarks)]
         for job in jobs:
             res = job.result()
             outs += res if isinstance(res, list) else [res]

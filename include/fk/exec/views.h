@@ -89,6 +89,17 @@ struct ViewOf<Read<PerThreadRead<ND::_2D, T>>> {
     }
 };
 
+// a 1-D buffer is one row
+template <typename T>
+struct ViewOf<Read<PerThreadRead<ND::_1D, T>>> {
+    static constexpr bool supported = true;
+    using type = PlainView<T>;
+    static type make(const Read<PerThreadRead<ND::_1D, T>>& iOp) {
+        const int n = static_cast<int>(iOp.params.dims.width);
+        return type{ iOp.params.data, 0u, n, 1, 0, 0, n, 1 };
+    }
+};
+
 template <PixelFormat PF>
 struct ViewOf<Read<ReadYUV<PF>>> {
     static constexpr bool supported = true;
@@ -256,6 +267,12 @@ struct OutOf<Write<PerThreadWrite<ND::_2D, O>>> {
     static constexpr bool supported = true;
     using type = PackedOut<O>;
     static type make(const Write<PerThreadWrite<ND::_2D, O>>& iOp) { return type{ iOp.params.data, iOp.params.dims.pitch, 0 }; }
+};
+template <typename O>
+struct OutOf<Write<PerThreadWrite<ND::_1D, O>>> {
+    static constexpr bool supported = true;
+    using type = PackedOut<O>;
+    static type make(const Write<PerThreadWrite<ND::_1D, O>>& iOp) { return type{ iOp.params.data, 0u, 0 }; }
 };
 template <typename O>
 struct OutOf<Write<PerThreadWrite<ND::_3D, O>>> {

@@ -7,6 +7,7 @@
 #include "fk/ops/yuv.h"
 #include "fk/ops/border_reader.h"
 #include "fk/ops/warping.h"
+#include "fk/ops/static_loop.h"
 
 namespace fk {
 

@@ -79,6 +79,13 @@ public:
     FK_HD_STATIC void exec(const Point& thread, const InputType& input, const OperationDataType& opData) { exec(thread, input, opData.params); }
     FK_HD_STATIC uint num_elems_x(const Point&, const OperationDataType& opData) { return opData.params.dims.width; }
     FK_HD_STATIC uint pitch(const Point&, const OperationDataType& opData) { return opData.params.dims.pitch; }
+    // one write per buffer (memory_operations.h:113-152: the batch builders of a write return the array itself)
+    template <size_t BATCH_N, typename Buffer>
+    static inline std::array<InstantiableType, BATCH_N> build_batch(const std::array<Buffer, BATCH_N>& buffers) {
+        std::array<InstantiableType, BATCH_N> out{};
+        for (size_t i = 0; i < BATCH_N; ++i) out[i] = build(buffers[i]);
+        return out;
+    }
     FK_HD_STATIC InstantiableType build(const ParamsType& params) { return InstantiableType{ { params } }; }
     FK_HD_STATIC InstantiableType build(const OperationDataType& opData) { return InstantiableType{ opData }; }
     static inline InstantiableType build(const Ptr<D, T>& ptr) { return build(ptr.ptr()); }
