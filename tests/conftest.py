@@ -19,6 +19,7 @@ def native_build():
     import fusedkernellibrary_amd as lib
     from fusedkernellibrary_amd import build
     wanted = list(lib.library_paths()) + [os.path.join(ROOT, "tests", "cpp", n) for n in ("conformance", "readme_dropin", "api_gpu")]
+    wanted.append(os.path.join(ROOT, "fusedkernellibrary_amd", "benchmarks", "reference_sweeps"))
     if not all(os.path.exists(p) for p in wanted):
         build.build_all()
     return wanted

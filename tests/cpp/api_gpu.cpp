@@ -1,5 +1,5 @@
 // The rest of the executeOperations surface on the GPU, as user code: buffer overloads (fused_kernel.h:26-54 of the
-// reference), conditional batches with a default value (batch_operations.h:234-241), 1-D and 3-D reads (generic kernel),
+// reference), conditional batches with a default value (batch_operations.h:234-241), 1-D reads (one long row of the pointwise kernel) with StaticLoop, 3-D reads (generic kernel),
 // cropped buffer views, the thread-fusion tag, setTo, stream sharing and error reporting.  Self-checking: exit code 0.
 #include <fused_kernel/fused_kernel.h>
 #include <fused_kernel/algorithms/image_processing/saturate.h>
@@ -62,17 +62,25 @@ int main() {
             for (uint x = 0; x < 1237; ++x) ok = ok && out.at(x, y) == static_cast<float>(in.at(x, y)) + 0.5f;
         EXPECT(ok);
     }
-    // 3. 1-D buffers (generic kernel) under the thread-fusion tag
-    {
-        Ptr1D<float> in(1000), out(1000);
-        for (uint i = 0; i < 1000; ++i) in.at(i) = 0.25f * static_cast<float>(i);
+    // 3. 1-D buffers under the thread-fusion tag; lengths that are and are not whole thread groups; StaticLoop
+    for (const uint n : { 1000u, 1003u, 1u, 262144u + 7u }) {
+        Ptr1D<float> in(n), out(n);
+        for (uint i = 0; i < n; ++i) in.at(i) = 0.25f * static_cast<float>(i % 4096u);
         Stream s2;
         in.upload(s2);
         executeOperations<TransformDPP<ParArch::GPU_AMD, TF::ENABLED>>(in, out, s2, Mul<float>::build(3.f), Sub<float>::build(1.f));
         out.download(s2);
         s2.sync();
         bool ok = true;
-        for (uint i = 0; i < 1000; ++i) ok = ok && out.at(i) == 0.25f * static_cast<float>(i) * 3.f - 1.f;
+        for (uint i = 0; i < n; ++i) ok = ok && out.at(i) == 0.25f * static_cast<float>(i % 4096u) * 3.f - 1.f;
+        EXPECT(ok);
+        // five additions in one operation; a loop of zero iterations still applies its operation once, as in the reference
+        executeOperations<TransformDPP<>>(s2, PerThreadRead<ND::_1D, float>::build(in), StaticLoop<Add<float>, 5>::build(0.5f),
+                                          StaticLoop<StaticLoop<Mul<float>, 2>, 0>::build(2.f), PerThreadWrite<ND::_1D, float>::build(out));
+        out.download(s2);
+        s2.sync();
+        ok = true;
+        for (uint i = 0; i < n; ++i) ok = ok && out.at(i) == (0.25f * static_cast<float>(i % 4096u) + 2.5f) * 4.f;
         EXPECT(ok);
     }
     // 4. 3-D read into a 3-D write, every plane (generic kernel), and getPlane views

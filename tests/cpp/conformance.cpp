@@ -147,6 +147,10 @@ static_assert(detail::border_index<BorderType::REFLECT>(-6, 8) == 5 && detail::b
               "the border diagrams of border_reader.h:26-33");
 static_assert(sizeof(WarpingParameters<WarpType::Affine>) == 32 && sizeof(WarpingParameters<WarpType::Perspective>) == 44);
 
+// StaticLoop (algorithms/basic_ops/static_loop.h:21-45 of the reference): N applications, at least one
+static_assert(StaticLoop<Add<int>, 5>::exec(1, 2) == 11 && StaticLoop<Add<int>, 1>::exec(1, 2) == 3 && StaticLoop<Add<int>, 0>::exec(1, 2) == 3);
+static_assert(StaticLoop<StaticLoop<Mul<int>, 3>, 2>::exec(1, 2) == 64 && isBinaryType<StaticLoop<Add<float>, 4>>);
+
 // DPP tags
 static_assert(TransformDPP<>::PAR_ARCH == ParArch::GPU_AMD && defaultParArch == ParArch::GPU_AMD && Stream::parArch() == ParArch::GPU_AMD);
 static_assert(exec::pixels_per_thread<float3, float3, false>() == 4 && exec::pixels_per_thread<uchar4, uchar, false>() == 4 &&

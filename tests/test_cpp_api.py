@@ -40,3 +40,15 @@ def test_executor_surface_as_user_code():
     assert os.path.exists(exe), "tests/cpp/api_gpu is not built"
     proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
     assert proc.returncode == 0 and "api_gpu ok" in proc.stdout, proc.stdout
+
+
+@pytest.mark.gpu
+def test_reference_benchmark_sweeps_run_and_check_themselves():
+    """The reference's four benchmark sweeps as user code (two timed iterations here): every sweep point compares its two
+    variants with each other and with the closed-form result, and the program exits non-zero on any mismatch."""
+    import json
+    exe = os.path.join(os.path.dirname(HERE), "fusedkernellibrary_amd", "benchmarks", "reference_sweeps")
+    assert os.path.exists(exe), "benchmarks/reference_sweeps is not built (python -m fusedkernellibrary_amd.build)"
+    proc = subprocess.run([exe, "all", "2"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=110)
+    rows = [json.loads(line) for line in proc.stdout.splitlines() if line.startswith("{")]
+    assert proc.returncode == 0 and len(rows) == 155 and all(r["passed"] for r in rows), proc.stdout[-2000:]
