@@ -57,7 +57,12 @@ CAPI_SIGNATURES = {
     "fk_yuv_crop_resize_norm_split": [_i, _i, _i, _vp, _sz, _i, _i, Rect, _i, _i, _f, _vp, _vp],
     "fk_border_crop_u8c3": [_i, _vp, _i, _i, _sz, _i, _i, _i, _i, C.POINTER(C.c_uint8), _vp, _sz, _vp],
     "fk_warp_u8c3_f32c3": [_i, C.POINTER(C.c_float), _vp, _i, _i, _sz, _i, _i, _vp, _sz, _vp],
+    "fk_tensor_relayout_f32c3": [_i, _vp, _i, _i, _i, _vp, _vp],
+    "fk_circular_tensor_read_f32c3": [_i, _i, _vp, _i, _i, _i, _vp, _vp],
+    "fk_circular_tensor_update_u8c3_split_f32": [_vp, _i, _i, _sz, _f, _vp, _vp, _i, _i, _i, _vp],
 }
+PACKED_TO_SPLIT, PACKED_TO_TRANSPOSED, SPLIT_TO_PACKED, TRANSPOSED_TO_PACKED = 0, 1, 2, 3
+ASCENDENT, DESCENDENT = 0, 1
 BORDER_CONSTANT, BORDER_REPLICATE, BORDER_REFLECT, BORDER_WRAP, BORDER_REFLECT_101 = 0, 1, 2, 3, 4
 WARP_AFFINE, WARP_PERSPECTIVE = 0, 1
 # PixelFormat / ColorRange / ColorPrimitives values of include/fk_capi.h
@@ -365,3 +370,38 @@ def warp_u8c3_f32c3(warp_type, matrix, src, out, stream=None, defer=False):
     m = (C.c_float * len(flat))(*flat)
     _deferred = _call(capi.fk_warp_u8c3_f32c3, (warp_type, m, p, w, h, pitch, dw, dh, q, out_pitch, _stream(stream)), defer)
     return _deferred if defer else out
+
+
+# ---- tensor layouts and circular tensors ------------------------------------------------------------------------------
+
+def tensor_relayout_f32c3(mode, src, w, h, planes, out, stream=None, defer=False):
+    """src / out: contiguous float32 tensors of planes*h*w*3 elements in the layouts the mode names."""
+    _, capi = load()
+    src, out = _dev(src, "float32"), _dev(out, "float32")
+    assert src.is_contiguous() and out.is_contiguous() and src.numel() == out.numel() == planes * h * w * 3
+    _deferred = _call(capi.fk_tensor_relayout_f32c3, (mode, C.c_void_p(src.data_ptr()), w, h, planes, C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def circular_tensor_read_f32c3(direction, first, ring, out, stream=None, defer=False):
+    """ring / out: (planes, h, w, 3) float32 contiguous."""
+    _, capi = load()
+    ring, out = _dev(ring, "float32"), _dev(out, "float32")
+    planes, h, w, _ = ring.shape
+    assert ring.is_contiguous() and out.is_contiguous() and out.shape == ring.shape
+    _deferred = _call(capi.fk_circular_tensor_read_f32c3, (direction, first, C.c_void_p(ring.data_ptr()), w, h, planes, C.c_void_p(out.data_ptr()),
+                                                          _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def circular_tensor_update_u8c3_split_f32(frame, mul_v, tensor, ring, next_index, newest_first, stream=None, defer=False):
+    """frame: (h, w, 3) uint8; tensor, ring: (batch, 3, h, w) float32 contiguous, updated in place.  Returns the ring
+    slot for the next update."""
+    _, capi = load()
+    p, w, h, pitch = _image(frame, "uint8")
+    tensor, ring = _dev(tensor, "float32"), _dev(ring, "float32")
+    batch = tensor.shape[0]
+    assert tensor.is_contiguous() and ring.is_contiguous() and tuple(tensor.shape) == tuple(ring.shape) == (batch, 3, h, w)
+    _deferred = _call(capi.fk_circular_tensor_update_u8c3_split_f32, (p, w, h, pitch, float(mul_v), C.c_void_p(tensor.data_ptr()), C.c_void_p(ring.data_ptr()),
+                                                                     batch, next_index, int(newest_first), _stream(stream)), defer)
+    return _deferred if defer else (next_index + 1) % batch

@@ -383,5 +383,33 @@ public:
     }
 };
 
+// A tensor whose channel planes are outermost: element (x, y, z) of channel c at
+// c*color_planes_pitch + z*plane_pitch + y*pitch + x (ptr_nd.h:104-126,696-714).
+template <typename T>
+class TensorT : public Ptr<ND::T3D, T> {
+public:
+    TensorT() {}
+    TensorT(const TensorT<T>& other) : Ptr<ND::T3D, T>(other) {}
+    TensorT(const Ptr<ND::T3D, T>& other) : Ptr<ND::T3D, T>(other) {}
+    TensorT(const uint& width_, const uint& height_, const uint& planes_, const uint& color_planes_ = 1,
+            const MemType& type_ = defaultMemType, const int& deviceID_ = 0)
+        : Ptr<ND::T3D, T>(tightDims(width_, height_, planes_, color_planes_), type_, deviceID_) {}
+    TensorT(T* data, const uint& width_, const uint& height_, const uint& planes_, const uint& color_planes_ = 1,
+            const MemType& type_ = MemType::Device, const int& deviceID_ = 0)
+        : Ptr<ND::T3D, T>(data, tightDims(width_, height_, planes_, color_planes_), type_, deviceID_) {}
+    TensorT& operator=(const TensorT&) = default;
+    void allocTensor(const uint& width_, const uint& height_, const uint& planes_, const uint& color_planes_ = 1,
+                     const MemType& type_ = defaultMemType, const int& deviceID_ = 0) {
+        this->allocPtr(tightDims(width_, height_, planes_, color_planes_), type_, deviceID_);
+    }
+
+private:
+    static PtrDims<ND::T3D> tightDims(uint w, uint h, uint planes, uint color_planes) {
+        PtrDims<ND::T3D> d(w, h, planes, color_planes);
+        detail::PtrLayout<ND::T3D, T>::tight(d);
+        return d;
+    }
+};
+
 } // namespace fk
 #endif

@@ -8,6 +8,7 @@
 #include "fk/ops/border_reader.h"
 #include "fk/ops/warping.h"
 #include "fk/ops/static_loop.h"
+#include "fk/ops/circular.h"
 
 namespace fk {
 

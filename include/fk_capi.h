@@ -138,6 +138,27 @@ int fk_border_crop_u8c3(int border_type, const void* src, int w, int h, size_t s
 int fk_warp_u8c3_f32c3(int warp_type, const float* matrix, const void* src, int w, int h, size_t src_pitch, int dst_w, int dst_h,
                        void* dst, size_t dst_pitch, void* stream);
 
+/* ---- tensor layouts and circular tensors ---------------------------------------------------------------------
+ * A tensor of `planes` images of h x w float3 pixels, rows tight: packed = planes, h, w, 3 (TensorRead / TensorWrite);
+ * split = planes, 3, h, w (TensorSplit / TensorPack); transposed = 3, planes, h, w (TensorTSplit / TensorTPack). */
+enum { FK_PACKED_TO_SPLIT = 0, FK_PACKED_TO_TRANSPOSED = 1, FK_SPLIT_TO_PACKED = 2, FK_TRANSPOSED_TO_PACKED = 3 };
+/* CircularDirection, core/execution_model/memory_operations.h:425 */
+enum { FK_ASCENDENT = 0, FK_DESCENDENT = 1 };
+
+/* TensorRead<float3> -> TensorSplit / TensorTSplit, or TensorPack / TensorTPack -> TensorWrite<float3>
+ * (memory_operations.h:195-348). */
+int fk_tensor_relayout_f32c3(int mode, const float* src, int w, int h, int planes, float* dst, void* stream);
+/* CircularTensorRead<direction, TensorRead<float3>, planes>{first} -> TensorWrite<float3> (memory_operations.h:527-566):
+ * plane z of dst is ring plane first + z (ascendent) or first - z (descendent) modulo planes; planes in 2, 3, 4, 8, 16. */
+int fk_circular_tensor_read_f32c3(int direction, int first, const float* ring, int w, int h, int planes, float* dst, void* stream);
+/* CircularTensor<float, 3, batch, order, ColorPlanes::Standard>::update(stream, PerThreadRead<_2D,uchar3>(frame),
+ * Cast<uchar3,float3>, Mul<float3>(mul_v), TensorSplit<float3>(tensor)) (core/data/circular_tensor.h:84-161) over memory
+ * the caller owns: `tensor` and `ring` are batch x 3 x h x w floats each; next_index is the ring slot this update fills
+ * (0 for the first update, then (next_index + 1) % batch).  After the call plane 0 (newest_first) or plane batch - 1 of
+ * `tensor` holds this frame and the other planes the previous frames by age.  batch in 2, 3, 4, 8, 16. */
+int fk_circular_tensor_update_u8c3_split_f32(const void* frame, int w, int h, size_t src_pitch, float mul_v, float* tensor, float* ring,
+                                             int batch, int next_index, int newest_first, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -24,6 +24,8 @@ BT601, BT709, BT2020 = 0, 1, 2
 BORDER_CONSTANT, BORDER_REPLICATE, BORDER_REFLECT, BORDER_WRAP, BORDER_REFLECT_101 = 0, 1, 2, 3, 4
 BORDER_TYPES = {"CONSTANT": 0, "REPLICATE": 1, "REFLECT": 2, "WRAP": 3, "REFLECT_101": 4}
 WARP_AFFINE, WARP_PERSPECTIVE = 0, 1
+PACKED_TO_SPLIT, PACKED_TO_TRANSPOSED, SPLIT_TO_PACKED, TRANSPOSED_TO_PACKED = 0, 1, 2, 3
+ASCENDENT, DESCENDENT = 0, 1
 YUV_MATRICES = [(RANGE_FULL, BT601), (RANGE_FULL, BT709), (RANGE_LIMITED, BT709), (RANGE_FULL, BT2020)]
 
 
@@ -85,12 +87,22 @@ def build(with_reference=True):
 class _Lib:
     """Thin numpy-facing wrapper; `ref=True` talks to the reference driver (literal host semantics)."""
 
-    def __init__(self, cdll, ref, yuv_cdll=None, bw_cdll=None):
+    def __init__(self, cdll, ref, yuv_cdll=None, bw_cdll=None, circ_cdll=None):
         self.c = cdll
         self.ref = ref
         self.yuv = yuv_cdll
         self.bw = bw_cdll
+        self.circ = circ_cdll
         pre = "fkr_" if ref else "fko_"
+        if circ_cdll is not None:
+            _v = C.c_void_p
+            fn = getattr(circ_cdll, pre + "tensor_relayout_f32c3")
+            fn.argtypes, fn.restype = [_i, _v, _i, _i, _i, _v], C.c_int
+            fn = getattr(circ_cdll, pre + "circular_tensor_read_f32c3")
+            fn.argtypes, fn.restype = [_i, _i, _v, _i, _i, _i, _v], C.c_int
+            if not ref:
+                fn = circ_cdll.fko_circular_tensor_update_u8c3_split_f32
+                fn.argtypes, fn.restype = [_v, _i, _i, _sz, _f, _v, _v, _i, _i, _i], C.c_int
         if bw_cdll is not None:
             _v = C.c_void_p
             fn = getattr(bw_cdll, pre + "border_crop_u8c3")
@@ -344,6 +356,33 @@ class _Lib:
         return out
 
 
+    # ---- tensor layouts, circular reads, CircularTensor::update ----
+    def _circ_fn(self, name):
+        if self.circ is None:
+            raise RuntimeError("the circular checker library is not built")
+        return getattr(self.circ, ("fkr_" if self.ref else "fko_") + name)
+
+    def tensor_relayout_f32c3(self, mode, src, w, h, planes):
+        """src / result are flat float32 arrays of planes*h*w*3 elements in the layouts the mode names."""
+        src = np.ascontiguousarray(src, np.float32)
+        out = np.empty(planes * h * w * 3, np.float32)
+        self._check(self._circ_fn("tensor_relayout_f32c3")(mode, _p(src), w, h, planes, _p(out)))
+        return out
+
+    def circular_tensor_read_f32c3(self, direction, first, ring):
+        """ring: (planes, h, w, 3) float32 -> same shape, planes in logical order."""
+        planes, h, w, _ = ring.shape
+        out = np.empty_like(ring)
+        self._check(self._circ_fn("circular_tensor_read_f32c3")(direction, first, _p(ring), w, h, planes, _p(out)))
+        return out
+
+    def circular_tensor_update_u8c3_split_f32(self, frame, mul_v, tensor, ring, next_index, newest_first):
+        """Updates tensor and ring, both (batch, 3, h, w) float32, in place."""
+        h, w, _ = frame.shape
+        self._check(self.circ.fko_circular_tensor_update_u8c3_split_f32(_p(frame), w, h, frame.strides[0], float(mul_v), _p(tensor), _p(ring),
+                                                                       tensor.shape[0], next_index, int(newest_first)))
+
+
 _cache = {}
 
 
@@ -353,7 +392,7 @@ def oracle():
         if not os.path.exists(path):
             build(with_reference=False)
         cdll = C.CDLL(path)
-        _cache["o"] = _Lib(cdll, ref=False, yuv_cdll=cdll, bw_cdll=cdll)
+        _cache["o"] = _Lib(cdll, ref=False, yuv_cdll=cdll, bw_cdll=cdll, circ_cdll=cdll)
     return _cache["o"]
 
 
@@ -365,5 +404,7 @@ def reference():
         yuv = C.CDLL(yuv_path) if os.path.exists(yuv_path) else None
         bw_path = os.path.join(_HERE, "_ref", "libfkref_border_warp.so")
         bw = C.CDLL(bw_path) if os.path.exists(bw_path) else None
-        _cache["r"] = _Lib(C.CDLL(path), ref=True, yuv_cdll=yuv, bw_cdll=bw) if os.path.exists(path) else None
+        circ_path = os.path.join(_HERE, "_ref", "libfkref_circular.so")
+        circ = C.CDLL(circ_path) if os.path.exists(circ_path) else None
+        _cache["r"] = _Lib(C.CDLL(path), ref=True, yuv_cdll=yuv, bw_cdll=bw, circ_cdll=circ) if os.path.exists(path) else None
     return _cache["r"]
