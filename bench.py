@@ -197,6 +197,19 @@ def other_configs(fk, timer, steps, warmup, only=None):
         ms = time_launches(timer, lambda i: call_w2(), steps, warmup)
         record("W2_perspective_4k_to_1920x1080_f32c3", ms, 1920 * 1080, 1920 * 1080 * 4 * 3 + 1920 * 1080 * 12, "four taps per output pixel, 2x down-scaling: no tap is shared")
 
+    # R1: one update of a ring of eight 1080p frames kept as normalised float planes (new frame through the chain, seven planes re-ordered)
+    if want("R1_circular_tensor_update_8x1080p"):
+        batch, hh, ww = 8, 1080, 1920
+        frame_r = rnd_u8(hh, ww, 3)
+        tensor_r = torch.zeros((batch, 3, hh, ww), device="cuda")
+        ring_r = torch.zeros((batch, 3, hh, ww), device="cuda")
+        calls_r = [fk.circular_tensor_update_u8c3_split_f32(frame_r, 1 / 255., tensor_r, ring_r, i, 1, defer=True) for i in range(batch)]
+        ms = time_launches(timer, lambda i: calls_r[i % batch](), steps, warmup)
+        px = hh * ww
+        record("R1_circular_tensor_update_8x1080p", ms, batch * px, px * 3 + px * 12 * 2 + (batch - 1) * px * 12 * 2,
+               "frame read + its planes written to tensor and ring + seven planes copied from the ring")
+        del tensor_r, ring_r, calls_r
+
     # C5: four chains over one 8192x8192 uchar4 image in one launch
     if not want("C5_divergent4_8192x8192"):
         return res

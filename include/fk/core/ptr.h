@@ -291,9 +291,9 @@ public:
     T& at(const uint& x, const uint& y) { return at(Point(static_cast<int>(x), static_cast<int>(y))); }
     template <ND DIM = D, std::enable_if_t<DIM == ND::_2D || DIM == ND::_3D, int> = 0>
     T at(const uint& x, const uint& y) const { return at(Point(static_cast<int>(x), static_cast<int>(y))); }
-    template <ND DIM = D, std::enable_if_t<DIM == ND::_3D, int> = 0>
+    template <ND DIM = D, std::enable_if_t<DIM == ND::_3D || DIM == ND::T3D, int> = 0>
     T& at(const uint& x, const uint& y, const uint& z) { return at(Point(static_cast<int>(x), static_cast<int>(y), static_cast<int>(z))); }
-    template <ND DIM = D, std::enable_if_t<DIM == ND::_3D, int> = 0>
+    template <ND DIM = D, std::enable_if_t<DIM == ND::_3D || DIM == ND::T3D, int> = 0>
     T at(const uint& x, const uint& y, const uint& z) const { return at(Point(static_cast<int>(x), static_cast<int>(y), static_cast<int>(z))); }
 
     // One image of a 3-D buffer as a 2-D buffer sharing ownership (ptr_nd.h:590-601).

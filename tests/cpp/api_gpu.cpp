@@ -177,7 +177,40 @@ int main() {
             }
         EXPECT(ok);
     }
-    // 7. a launch the runtime rejects surfaces as the reference's exception text
+    // 7. CircularTensor (owning its memory): the last four results of a chain in age order, in the three layouts
+    {
+        constexpr int B = 4;
+        constexpr uint W = 40, H = 12;
+        CircularTensor<float, 3, B, CircularTensorOrder::NewestFirst, ColorPlanes::Standard> newest_first(W, H);
+        CircularTensor<float, 3, B, CircularTensorOrder::OldestFirst, ColorPlanes::Transposed> transposed(W, H);
+        CircularTensor<float3, 1, B, CircularTensorOrder::OldestFirst, ColorPlanes::Standard> packed(W, H);
+        Ptr2D<uchar3> frame(W, H);
+        const auto read = PerThreadRead<ND::_2D, uchar3>::build(frame);
+        bool ok = true;
+        for (int k = 0; k < 7; ++k) {
+            setTo(uchar3{ static_cast<uchar>(k + 1), static_cast<uchar>(10 + k), static_cast<uchar>(100 + k) }, frame, stream);
+            newest_first.update(stream, read, Cast<uchar3, float3>::build(), Mul<float3>::build(make_set<float3>(2.f)), TensorSplit<float3>::build(newest_first.ptr()));
+            transposed.update(stream, read, Cast<uchar3, float3>::build(), TensorTSplit<float3>::build(transposed.ptr()));
+            packed.update(stream, read, Cast<uchar3, float3>::build(), TensorWrite<float3>::build(packed.ptr()));
+            newest_first.download(stream);
+            transposed.download(stream);
+            packed.download(stream);
+            stream.sync();
+            for (int age = 0; age <= (k < B - 1 ? k : B - 1); ++age) {
+                const float r = static_cast<float>(k - age + 1), g = static_cast<float>(10 + k - age), b = static_cast<float>(100 + k - age);
+                // split: channel planes of image `age` follow each other; at() addresses channel 0, the others are W*H further
+                const float* p = &newest_first.at(5, 3, static_cast<uint>(age));
+                ok = ok && p[0] == 2.f * r && p[W * H] == 2.f * g && p[2 * W * H] == 2.f * b;
+                const uint z = static_cast<uint>(B - 1 - age);
+                const float* t = &transposed.at(7, 2, z); // transposed: channel planes are outermost, B*W*H apart
+                ok = ok && t[0] == r && t[B * W * H] == g && t[2 * B * W * H] == b;
+                const float3 q = packed.at(W - 1, H - 1, z);
+                ok = ok && q.x == r && q.y == g && q.z == b;
+            }
+        }
+        EXPECT(ok && newest_first.nextUpdateIdx() == 7 % B);
+    }
+    // 8. a launch the runtime rejects surfaces as the reference's exception text
     {
         bool threw = false;
         try {

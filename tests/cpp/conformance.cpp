@@ -151,6 +151,19 @@ static_assert(sizeof(WarpingParameters<WarpType::Affine>) == 32 && sizeof(Warpin
 static_assert(StaticLoop<Add<int>, 5>::exec(1, 2) == 11 && StaticLoop<Add<int>, 1>::exec(1, 2) == 3 && StaticLoop<Add<int>, 0>::exec(1, 2) == 3);
 static_assert(StaticLoop<StaticLoop<Mul<int>, 3>, 2>::exec(1, 2) == 64 && isBinaryType<StaticLoop<Add<float>, 4>>);
 
+// circular memory operations and CircularTensor (memory_operations.h:425-443, circular_tensor.h:24-61 of the reference)
+static_assert(circular_batch_internal::computeCircularThreadIdx<CircularDirection::Ascendent, 4>(Point(1, 2, 3), 2).z == 1 &&
+              circular_batch_internal::computeCircularThreadIdx<CircularDirection::Descendent, 4>(Point(1, 2, 3), 2).z == 3 &&
+              circular_batch_internal::computeCircularThreadIdx<CircularDirection::Descendent, 4>(Point(1, 2, 1), 2).z == 1);
+static_assert(SequenceSelectorType<CircularTensorOrder::NewestFirst, 4>::at(0) == 1 && SequenceSelectorType<CircularTensorOrder::NewestFirst, 4>::at(3) == 2 &&
+              SequenceSelectorType<CircularTensorOrder::OldestFirst, 4>::at(3) == 1 && SequenceSelectorType<CircularTensorOrder::OldestFirst, 4>::at(0) == 2);
+static_assert(CTReadDirection_v<CircularTensorOrder::NewestFirst> == CircularDirection::Descendent &&
+              std::is_same_v<CircularTensorStoreType<float, 3>::type, float3> && std::is_same_v<CircularTensorStoreType<uchar4, 1>::type, uchar4> &&
+              std::is_base_of_v<TensorT<float>, CircularTensor<float, 3, 4, CircularTensorOrder::OldestFirst, ColorPlanes::Transposed>>);
+static_assert(isWriteType<Write<TensorTSplit<float3>>> && isReadType<Read<TensorPack<float3>>> && isReadType<Read<TensorTPack<uchar4>>> &&
+              isReadType<Read<CircularTensorRead<CircularDirection::Ascendent, TensorRead<float3>, 4>>> &&
+              isWriteType<Write<CircularBatchWrite<CircularDirection::Ascendent, PerThreadWrite<ND::_2D, float>, 4>>>);
+
 // DPP tags
 static_assert(TransformDPP<>::PAR_ARCH == ParArch::GPU_AMD && defaultParArch == ParArch::GPU_AMD && Stream::parArch() == ParArch::GPU_AMD);
 static_assert(exec::pixels_per_thread<float3, float3, false>() == 4 && exec::pixels_per_thread<uchar4, uchar, false>() == 4 &&
