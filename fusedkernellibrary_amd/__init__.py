@@ -57,6 +57,7 @@ CAPI_SIGNATURES = {
     "fk_yuv_crop_resize_norm_split": [_i, _i, _i, _vp, _sz, _i, _i, Rect, _i, _i, _f, _vp, _vp],
     "fk_border_crop_u8c3": [_i, _vp, _i, _i, _sz, _i, _i, _i, _i, C.POINTER(C.c_uint8), _vp, _sz, _vp],
     "fk_warp_u8c3_f32c3": [_i, C.POINTER(C.c_float), _vp, _i, _i, _sz, _i, _i, _vp, _sz, _vp],
+    "fk_deinterlace_u8c3_f32c3": [_i, _i, _vp, _i, _i, _sz, _vp, _sz, _vp],
     "fk_tensor_relayout_f32c3": [_i, _vp, _i, _i, _i, _vp, _vp],
     "fk_circular_tensor_read_f32c3": [_i, _i, _vp, _i, _i, _i, _vp, _vp],
     "fk_circular_tensor_update_u8c3_split_f32": [_vp, _i, _i, _sz, _f, _vp, _vp, _i, _i, _i, _vp],
@@ -65,6 +66,7 @@ PACKED_TO_SPLIT, PACKED_TO_TRANSPOSED, SPLIT_TO_PACKED, TRANSPOSED_TO_PACKED = 0
 ASCENDENT, DESCENDENT = 0, 1
 BORDER_CONSTANT, BORDER_REPLICATE, BORDER_REFLECT, BORDER_WRAP, BORDER_REFLECT_101 = 0, 1, 2, 3, 4
 WARP_AFFINE, WARP_PERSPECTIVE = 0, 1
+DEINTERLACE_BLEND, DEINTERLACE_INTER_LINEAR = 0, 1
 # PixelFormat / ColorRange / ColorPrimitives values of include/fk_capi.h
 NV12, NV21, P010, P210, Y210, UYVY = 0, 1, 3, 6, 8, 10
 RANGE_LIMITED, RANGE_FULL = 0, 1
@@ -369,6 +371,16 @@ def warp_u8c3_f32c3(warp_type, matrix, src, out, stream=None, defer=False):
         raise FkError("matrix must be 2x3 (affine) or 3x3 (perspective)")
     m = (C.c_float * len(flat))(*flat)
     _deferred = _call(capi.fk_warp_u8c3_f32c3, (warp_type, m, p, w, h, pitch, dw, dh, q, out_pitch, _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def deinterlace_u8c3_f32c3(kind, use_even_lines, src, out, stream=None, defer=False):
+    """src: (h, w, 3) uint8; out: (h, w, 3) float32."""
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    q, ow, oh, out_pitch = _image(out, "float32")
+    assert (ow, oh) == (w, h)
+    _deferred = _call(capi.fk_deinterlace_u8c3_f32c3, (kind, int(use_even_lines), p, w, h, pitch, q, out_pitch, _stream(stream)), defer)
     return _deferred if defer else out
 
 

@@ -1,4 +1,4 @@
-// fk_capi_border_warp.hip — the BorderReader and Warping entry points of include/fk_capi.h, built with the fk::
+// fk_capi_border_warp.hip — the BorderReader, Warping and Deinterlace entry points of include/fk_capi.h, built with the fk::
 // operator API and handed to executeOperations.  Compiled by hipcc into libfk_capi.so.
 #include "fk_capi_common.h"
 
@@ -65,6 +65,27 @@ int fk_warp_u8c3_f32c3(int warp_type, const float* matrix, const void* src, int 
         if (warp_type == FK_WARP_AFFINE) warp<WarpType::Affine>(s, matrix, src, w, h, src_pitch, dst_w, dst_h, dst, dst_pitch);
         else if (warp_type == FK_WARP_PERSPECTIVE) warp<WarpType::Perspective>(s, matrix, src, w, h, src_pitch, dst_w, dst_h, dst, dst_pitch);
         else return unsupported("warp type must be affine or perspective");
+        return FK_OK;
+    });
+}
+
+int fk_deinterlace_u8c3_f32c3(int type, int use_even_lines, const void* src, int w, int h, size_t src_pitch, void* dst, size_t dst_pitch,
+                              void* stream) {
+    if (src == nullptr || dst == nullptr) return bad_argument("null pointer");
+    if (w <= 0 || h <= 0) return bad_argument("empty image");
+    if (src_pitch < static_cast<size_t>(w) * 3 || dst_pitch < static_cast<size_t>(w) * 12) return bad_argument("pitch shorter than a row");
+    return guarded([&]() -> int {
+        Stream s(stream);
+        const auto read = PerThreadRead<ND::_2D, uchar3>::build(view2d<uchar3>(src, w, h, src_pitch));
+        const auto write = PerThreadWrite<ND::_2D, float3>::build(view2d<float3>(dst, w, h, dst_pitch));
+        if (type == FK_DEINTERLACE_BLEND) {
+            executeOperations<TransformDPP<>>(s, read.then(Deinterlace<DeinterlaceType::BLEND>::build()), write);
+        } else if (type == FK_DEINTERLACE_INTER_LINEAR) {
+            const DeinterlaceParameters<DeinterlaceType::INTER_LINEAR> params{ use_even_lines != 0 };
+            executeOperations<TransformDPP<>>(s, read.then(Deinterlace<DeinterlaceType::INTER_LINEAR>::build(params)), write);
+        } else {
+            return unsupported("deinterlace type must be BLEND or INTER_LINEAR");
+        }
         return FK_OK;
     });
 }

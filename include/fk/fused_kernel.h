@@ -9,6 +9,7 @@
 #include "fk/ops/warping.h"
 #include "fk/ops/static_loop.h"
 #include "fk/ops/circular.h"
+#include "fk/ops/deinterlace.h"
 
 namespace fk {
 

@@ -28,10 +28,12 @@ enum class ColorDepth { p8bit = 0, p10bit = 1, p12bit = 2, f24bit = 3 };
 
 // CCIR 601 luma of the first three channels as stored, rounded to nearest even for integer outputs
 // (color_conversion.h:47-77).
-template <typename I, typename O = VBase<I>>
+enum class GrayFormula { CCIR_601 };
+
+template <typename I, typename O = VBase<I>, GrayFormula GF = GrayFormula::CCIR_601>
 struct RGB2Gray {
 private:
-    using SelfType = RGB2Gray<I, O>;
+    using SelfType = RGB2Gray<I, O, GF>;
 
 public:
     FK_UNARY_OPERATION(RGB2Gray, I, O)
@@ -63,6 +65,19 @@ public:
                                                                       : static_cast<VBase<I>>(4095);
         return O4{ input.x, input.y, input.z, alpha };
     }
+};
+
+// A given alpha appended to a 3-channel pixel (color_conversion.h:29-40).
+template <typename I, VBase<I> alpha>
+struct StaticAddAlpha {
+private:
+    using SelfType = StaticAddAlpha<I, alpha>;
+    using O4 = VectorType_t<VBase<I>, 4>;
+
+public:
+    FK_UNARY_OPERATION(StaticAddAlpha, I, O4)
+    static_assert(cn<I> == 3, "StaticAddAlpha takes a 3-channel pixel");
+    FK_HD_STATIC OutputType exec(const InputType& input) { return O4{ input.x, input.y, input.z, alpha }; }
 };
 
 namespace detail {

@@ -138,6 +138,14 @@ int fk_border_crop_u8c3(int border_type, const void* src, int w, int h, size_t s
 int fk_warp_u8c3_f32c3(int warp_type, const float* matrix, const void* src, int w, int h, size_t src_pitch, int dst_w, int dst_h,
                        void* dst, size_t dst_pitch, void* stream);
 
+/* DeinterlaceType, algorithms/image_processing/deinterlace.h:25 */
+enum { FK_DEINTERLACE_BLEND = 0, FK_DEINTERLACE_INTER_LINEAR = 1 };
+/* PerThreadRead<_2D,uchar3> -> Deinterlace<type>(use_even_lines) -> PerThreadWrite<_2D,float3> (deinterlace.h:41-126):
+ * BLEND averages each line with the one above; INTER_LINEAR keeps the even (use_even_lines != 0) or odd lines and
+ * rebuilds the others from their two neighbours.  Sums are integer, + 1, times 0.5f. */
+int fk_deinterlace_u8c3_f32c3(int type, int use_even_lines, const void* src, int w, int h, size_t src_pitch, void* dst, size_t dst_pitch,
+                              void* stream);
+
 /* ---- tensor layouts and circular tensors ---------------------------------------------------------------------
  * A tensor of `planes` images of h x w float3 pixels, rows tight: packed = planes, h, w, 3 (TensorRead / TensorWrite);
  * split = planes, 3, h, w (TensorSplit / TensorPack); transposed = 3, planes, h, w (TensorTSplit / TensorTPack). */

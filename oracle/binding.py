@@ -24,6 +24,7 @@ BT601, BT709, BT2020 = 0, 1, 2
 BORDER_CONSTANT, BORDER_REPLICATE, BORDER_REFLECT, BORDER_WRAP, BORDER_REFLECT_101 = 0, 1, 2, 3, 4
 BORDER_TYPES = {"CONSTANT": 0, "REPLICATE": 1, "REFLECT": 2, "WRAP": 3, "REFLECT_101": 4}
 WARP_AFFINE, WARP_PERSPECTIVE = 0, 1
+DEINTERLACE_BLEND, DEINTERLACE_INTER_LINEAR = 0, 1
 PACKED_TO_SPLIT, PACKED_TO_TRANSPOSED, SPLIT_TO_PACKED, TRANSPOSED_TO_PACKED = 0, 1, 2, 3
 ASCENDENT, DESCENDENT = 0, 1
 YUV_MATRICES = [(RANGE_FULL, BT601), (RANGE_FULL, BT709), (RANGE_LIMITED, BT709), (RANGE_FULL, BT2020)]
@@ -109,6 +110,8 @@ class _Lib:
             fn.argtypes, fn.restype = [_i, _v, _i, _i, _sz, _i, _i, _i, _i, _v, _v, _sz], C.c_int
             fn = getattr(bw_cdll, pre + "warp_coords")
             fn.argtypes, fn.restype = [_i, _v, _i, _i, _v], None
+            fn = getattr(bw_cdll, pre + "deinterlace_u8c3_f32c3")
+            fn.argtypes, fn.restype = [_i, _i, _v, _i, _i, _sz, _v, _sz], C.c_int
             fn = getattr(bw_cdll, pre + "warp_u8c3_f32c3")
             fn.argtypes, fn.restype = [_i, _v, _v, _i, _i, _sz, _i, _i] + ([] if ref else [_i]) + [_v, _sz], C.c_int
             if not ref:
@@ -355,6 +358,12 @@ class _Lib:
         self._check(self._bw_fn("warp_u8c3_f32c3")(*args, _p(out), out.strides[0]))
         return out
 
+
+    def deinterlace_u8c3_f32c3(self, kind, use_even_lines, src):
+        h, w, _ = src.shape
+        out = np.empty((h, w, 3), np.float32)
+        self._check(self._bw_fn("deinterlace_u8c3_f32c3")(kind, int(use_even_lines), _p(src), w, h, src.strides[0], _p(out), out.strides[0]))
+        return out
 
     # ---- tensor layouts, circular reads, CircularTensor::update ----
     def _circ_fn(self, name):

@@ -10,6 +10,10 @@
  *     with quirk = 0: identity and integer translations (the output is the shifted image), agreement with the
  *     literal result wherever floor(x) == floor(y), the pure-scaling affine warp against the separately pinned
  *     resize sample fko_bilinear_u8, and a double-precision evaluation.
+ *   - fko_deinterlace_u8c3_f32c3: the BLEND known answers of the reference's own unit test
+ *     (utests/algorithm/image_processing/utest_deinterlace.h:24-45; its INTER_LINEAR tables hold the truncated
+ *     values 2 and 1 where the operation's code yields 2.5 and 1.5, and the code is what is followed), oracle/_ref
+ *     on random images, and closed forms (constant image, kept lines unchanged, numpy averages).
  */
 #include "fk_oracle_border_warp.h"
 
@@ -90,6 +94,34 @@ int fko_warp_u8c3_f32c3(int warp_type, const float* matrix, const uint8_t* src, 
             } else {
                 o[0] = o[1] = o[2] = 0.f;
             }
+        }
+    }
+    return 0;
+}
+
+/* Deinterlace::exec, deinterlace.h:53-126: integer sums of the promoted channels, + 1, times 0.5f */
+int fko_deinterlace_u8c3_f32c3(int type, int use_even_lines, const uint8_t* src, int w, int h, size_t src_pitch, float* dst,
+                               size_t dst_pitch) {
+    if (type != FKO_DEINTERLACE_BLEND && type != FKO_DEINTERLACE_INTER_LINEAR) return 1;
+    for (int y = 0; y < h; ++y) {
+        const uint8_t* cur = src + (size_t)y * src_pitch;
+        const uint8_t* above = y > 0 ? cur - src_pitch : cur;
+        const uint8_t* below = y + 1 < h ? cur + src_pitch : cur;
+        float* out = (float*)((char*)dst + (size_t)y * dst_pitch);
+        int mode; /* 0 pass through, 1 current + above, 2 above + below */
+        if (type == FKO_DEINTERLACE_BLEND) {
+            mode = y > 0 ? 1 : 0; /* :97-104 */
+        } else {                  /* :118-125 */
+            const int odd = y & 1;
+            /* the last line never interpolates: for an odd number of lines the reference's USE_ODD case reads the line
+             * past the image there (it assumes an even number, deinterlace.h:112) */
+            const int interpolate = y != h - 1 && (use_even_lines ? odd : (!odd && y != 0));
+            mode = interpolate ? 2 : 0;
+        }
+        for (int i = 0; i < 3 * w; ++i) {
+            if (mode == 0) out[i] = (float)cur[i] * 1.f;
+            else if (mode == 1) out[i] = (float)((int)cur[i] + (int)above[i] + 1) * 0.5f;
+            else out[i] = (float)((int)above[i] + (int)below[i] + 1) * 0.5f;
         }
     }
     return 0;

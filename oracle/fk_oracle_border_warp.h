@@ -1,4 +1,5 @@
-/* fk_oracle_border_warp.h — CPU restatement of BorderReader and Warping on the Fused Kernel Library's Transform path.
+/* fk_oracle_border_warp.h — CPU restatement of BorderReader, Warping and Deinterlace on the Fused Kernel Library's
+ * Transform path.
  *
  * TEST INFRASTRUCTURE ONLY (see fk_oracle.h): the checker the GPU library is compared with; nothing in the shipped
  * library links, loads or calls it.  Plain C, FP32 in the reference's evaluation order, no FMA contraction.
@@ -28,6 +29,12 @@ void fko_warp_coords(int warp_type, const float* matrix, int x, int y, float out
 /* PerThreadRead<_2D,uchar3> -> Warping<type>(matrix, dst size) -> PerThreadWrite<_2D,float3> */
 int fko_warp_u8c3_f32c3(int warp_type, const float* matrix, const uint8_t* src, int w, int h, size_t src_pitch,
                         int dst_w, int dst_h, int quirk_y1_from_x, float* dst, size_t dst_pitch);
+
+/* DeinterlaceType, algorithms/image_processing/deinterlace.h:25 */
+enum { FKO_DEINTERLACE_BLEND = 0, FKO_DEINTERLACE_INTER_LINEAR = 1 };
+/* PerThreadRead<_2D,uchar3> -> Deinterlace<type>(use_even_lines) -> PerThreadWrite<_2D,float3> */
+int fko_deinterlace_u8c3_f32c3(int type, int use_even_lines, const uint8_t* src, int w, int h, size_t src_pitch, float* dst,
+                               size_t dst_pitch);
 
 #ifdef __cplusplus
 }

@@ -7,6 +7,7 @@
 #include <fused_kernel/core/execution_model/memory_operations.h>
 #include <fused_kernel/algorithms/image_processing/border_reader.h>
 #include <fused_kernel/algorithms/image_processing/crop.h>
+#include <fused_kernel/algorithms/image_processing/deinterlace.h>
 #include <fused_kernel/algorithms/image_processing/warping.h>
 #include <fused_kernel/fused_kernel.h>
 
@@ -94,6 +95,21 @@ int fkr_warp_u8c3_f32c3(int warp_type, const float* matrix, const uint8_t* src, 
     if (warp_type == FKO_WARP_AFFINE) warp<WarpType::Affine>(matrix, src, w, h, src_pitch, dst_w, dst_h, dst, dst_pitch);
     else if (warp_type == FKO_WARP_PERSPECTIVE) warp<WarpType::Perspective>(matrix, src, w, h, src_pitch, dst_w, dst_h, dst, dst_pitch);
     else return 1;
+    return 0;
+}
+
+int fkr_deinterlace_u8c3_f32c3(int type, int use_even_lines, const uint8_t* src, int w, int h, size_t src_pitch, float* dst, size_t dst_pitch) {
+    Stream_<ParArch::CPU> stream;
+    const auto read = PerThreadRead<ND::_2D, uchar3>::build(raw2d<uchar3>(src, w, h, src_pitch));
+    const auto write = PerThreadWrite<ND::_2D, float3>::build(raw2d<float3>(dst, w, h, dst_pitch));
+    if (type == FKO_DEINTERLACE_BLEND) {
+        executeOperations<CPU>(stream, read.then(Deinterlace<DeinterlaceType::BLEND>::build()), write);
+    } else if (type == FKO_DEINTERLACE_INTER_LINEAR) {
+        const DeinterlaceParameters<DeinterlaceType::INTER_LINEAR> params{ use_even_lines != 0 };
+        executeOperations<CPU>(stream, read.then(Deinterlace<DeinterlaceType::INTER_LINEAR>::build(params)), write);
+    } else {
+        return 1;
+    }
     return 0;
 }
 

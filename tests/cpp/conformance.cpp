@@ -164,6 +164,28 @@ static_assert(isWriteType<Write<TensorTSplit<float3>>> && isReadType<Read<Tensor
               isReadType<Read<CircularTensorRead<CircularDirection::Ascendent, TensorRead<float3>, 4>>> &&
               isWriteType<Write<CircularBatchWrite<CircularDirection::Ascendent, PerThreadWrite<ND::_2D, float>, 4>>>);
 
+// known answers of the reference's unit tests for single operations (utests/algorithm/image_processing/
+// utest_color_conversion.h:34-224; where its harness compares one channel, x, the values of that channel)
+static_assert(IsEven<uint>::exec(0u) && !IsEven<uint>::exec(1u) && IsEven<uint>::exec(2u) && !IsEven<uint>::exec(3u));
+static_assert(AddOpaqueAlpha<uchar3, ColorDepth::p8bit>::exec(uchar3{ 100, 150, 200 }).w == 255 && AddOpaqueAlpha<uchar3, ColorDepth::p8bit>::exec(uchar3{ 50, 75, 125 }).x == 50 &&
+              StaticAddAlpha<uchar3, 255>::exec(uchar3{ 100, 150, 200 }).w == 255 && StaticAddAlpha<uchar3, 7>::exec(uchar3{ 50, 75, 125 }).w == 7);
+static_assert(ColorConversion<ColorConversionCodes::COLOR_BGR2BGRA, uchar3, uchar4>::exec(uchar3{ 100, 150, 200 }).z == 200 &&
+              ColorConversion<ColorConversionCodes::COLOR_BGR2BGRA, uchar3, uchar4>::exec(uchar3{ 100, 150, 200 }).w == 255 &&
+              ColorConversion<ColorConversionCodes::COLOR_BGR2RGB, uchar3, uchar3>::exec(uchar3{ 100, 150, 200 }).x == 200 &&
+              ColorConversion<ColorConversionCodes::COLOR_BGR2RGB, uchar3, uchar3>::exec(uchar3{ 50, 75, 125 }).z == 50);
+static_assert(DenormalizePixel<float3, ColorDepth::p8bit>::exec(float3{ 0.0f, 0.5f, 1.0f }).y == 127.5f && DenormalizePixel<float3, ColorDepth::p8bit>::exec(float3{ 0.25f, 0.75f, 0.9f }).x == 63.75f &&
+              NormalizePixel<uchar3, ColorDepth::p8bit>::exec(uchar3{ 0, 128, 255 }).z == 1.0f && NormalizePixel<uchar3, ColorDepth::p8bit>::exec(uchar3{ 64, 192, 32 }).x == 64.0f / 255.0f &&
+              SaturateDenormalizePixel<float3, uchar3, ColorDepth::p8bit>::exec(float3{ -0.5f, 0.5f, 1.5f }).x == 0 &&
+              SaturateDenormalizePixel<float3, uchar3, ColorDepth::p8bit>::exec(float3{ 0.25f, 0.75f, 0.9f }).x == 63 &&
+              NormalizeColorRangeDepth<float3, ColorDepth::p8bit>::exec(float3{ 64.0f, 192.0f, 100.0f }).y == 192.0f);
+// Deinterlace builders (tests/algorithm/test_deinterlace.h:21-44 of the reference)
+constexpr auto kBlend = Deinterlace<DeinterlaceType::BLEND>::build(kRead);
+constexpr auto kLinear = Deinterlace<DeinterlaceType::INTER_LINEAR>::build(DeinterlaceLinear::USE_EVEN, kRead);
+static_assert(std::is_same_v<std::decay_t<decltype(kBlend)>, ReadBack<Deinterlace<DeinterlaceType::BLEND, Read<ReadU3>>>> &&
+              std::is_same_v<std::decay_t<decltype(kLinear)>, ReadBack<Deinterlace<DeinterlaceType::INTER_LINEAR, Read<ReadU3>>>> && kLinear.params.useEvenLines &&
+              std::is_same_v<std::decay_t<decltype(kRead.then(Deinterlace<DeinterlaceType::BLEND>::build()))>, std::decay_t<decltype(kBlend)>> &&
+              std::is_same_v<std::decay_t<decltype(kBlend)>::Operation::OutputType, float3>);
+
 // DPP tags
 static_assert(TransformDPP<>::PAR_ARCH == ParArch::GPU_AMD && defaultParArch == ParArch::GPU_AMD && Stream::parArch() == ParArch::GPU_AMD);
 static_assert(exec::pixels_per_thread<float3, float3, false>() == 4 && exec::pixels_per_thread<uchar4, uchar, false>() == 4 &&
@@ -171,6 +193,11 @@ static_assert(exec::pixels_per_thread<float3, float3, false>() == 4 && exec::pix
 
 int main() {
     int failures = 0;
+    // RGB2Gray known answers of the reference's unit test (rounding to nearest is not a constant expression)
+    EXPECT((RGB2Gray<uchar3, uchar>::exec(uchar3{ 255, 0, 0 }) == 76 && RGB2Gray<uchar3, uchar>::exec(uchar3{ 0, 255, 0 }) == 150 &&
+            RGB2Gray<uchar3, uchar>::exec(uchar3{ 0, 0, 255 }) == 29));
+    EXPECT((RGB2Gray<uchar3, uchar, GrayFormula::CCIR_601>::exec(uchar3{ 50, 100, 150 }) == 91 &&
+            RGB2Gray<uchar3, uchar, GrayFormula::CCIR_601>::exec(uchar3{ 75, 125, 200 }) == 119));
     // owning host buffers: refcount through copies, crop views share ownership, at() addresses by pitch
     {
         Ptr2D<uchar3> img(64, 32, 0, MemType::Host);

@@ -1,5 +1,5 @@
 """Writes tests/golden/reference_border_warp_vectors.npz from the REFERENCE's own headers
-(oracle/_ref/libfkref_border_warp.so, built by oracle/Makefile from /root/reference as it lies there; its CPU backend).
+(oracle/_ref/libfkref_border_warp.so: BorderReader, Warping and Deinterlace; built by oracle/Makefile from /root/reference as it lies there; its CPU backend).
 
 Run in the build container only: `python tests/golden/make_golden_border_warp.py`.  The fixture holds outputs only;
 inputs are regenerated from the seed and parameters below.  Nothing of the reference's source is stored.  The source
@@ -38,6 +38,8 @@ def main():
     for name, (wt, m, dst) in WARPS.items():
         out[f"warp_{name}"] = r.warp_u8c3_f32c3(wt, m, src, dst)
         out[f"coords_{name}"] = np.array([[r.warp_coords(wt, m, x, y) for x in range(0, dst[0], 5)] for y in range(0, dst[1], 5)], np.float32)
+    for kind, even in ((B.DEINTERLACE_BLEND, 1), (B.DEINTERLACE_INTER_LINEAR, 1), (B.DEINTERLACE_INTER_LINEAR, 0)):
+        out[f"deinterlace_{kind}_{even}"] = r.deinterlace_u8c3_f32c3(kind, even, src)  # 40 lines: an even number
     np.savez_compressed(os.path.join(HERE, "reference_border_warp_vectors.npz"), **out)
     print("wrote", len(out), "arrays")
 

@@ -123,3 +123,17 @@ def test_argument_errors(fk):
         fk.border_crop_u8c3(5, src, 1, 1, out_u8(10, 10))  # TRANSPARENT_: declared by the reference, not implemented there
     with pytest.raises(fk.FkError, match="unsupported"):
         fk.warp_u8c3_f32c3(2, [[1, 0, 0], [0, 1, 0], [0, 0, 1]], src, out_f32(8, 8))
+
+
+@pytest.mark.parametrize("kind,even", [(B.DEINTERLACE_BLEND, 1), (B.DEINTERLACE_INTER_LINEAR, 1), (B.DEINTERLACE_INTER_LINEAR, 0)])
+def test_deinterlace(fk, oracle, kind, even):
+    src = oracle.bytes(G.SEED, G.SRC)
+    out = out_f32(G.SRC[1], G.SRC[0])
+    fk.deinterlace_u8c3_f32c3(kind, even, dev(src), out)
+    assert same_bits(host(out), GOLD[f"deinterlace_{kind}_{even}"])
+    for i, ((w, h), pad) in enumerate((((1, 1), 0), ((8, 8), 0), ((33, 7), 3), ((1920, 1080), 0), ((720, 576), 4))):
+        img = oracle.bytes(500 + i, (h, w, 3))
+        out = out_f32(w, h, pad)
+        fk.deinterlace_u8c3_f32c3(kind, even, dev(img, pad), out)
+        torch.cuda.synchronize()
+        assert same_bits(host(out), oracle.deinterlace_u8c3_f32c3(kind, even, img)), (w, h)

@@ -166,3 +166,42 @@ def test_warp_canonical_against_literal_and_double(oracle):
                 ref = (src[y1, x1] * (1 - fx) * (1 - fy) + src[y1, x2] * fx * (1 - fy) + src[y2, x1] * (1 - fx) * fy + src[y2, x2] * fx * fy)
                 np.testing.assert_allclose(can[y, x], ref, rtol=1e-4, atol=0.35)
         assert checked >= 3
+
+
+# ---- Deinterlace --------------------------------------------------------------------------------------------------------------
+def test_deinterlace_known_answers_and_golden(oracle):
+    # the BLEND table of the reference's own unit test (utests/algorithm/image_processing/utest_deinterlace.h:24-45):
+    # lines alternate (2, 4, 8) and (1, 1, 1); every line but the first becomes (2, 3, 5)
+    src = np.empty((8, 8, 3), np.uint8)
+    src[0::2] = (2, 4, 8)
+    src[1::2] = (1, 1, 1)
+    want = np.empty((8, 8, 3), np.float32)
+    want[0] = (2, 4, 8)
+    want[1:] = (2, 3, 5)
+    assert same_bits(oracle.deinterlace_u8c3_f32c3(B.DEINTERLACE_BLEND, 1, src), want)
+    # INTER_LINEAR on the same image, from the operation's code: kept lines unchanged, rebuilt lines (a + b + 1) * 0.5
+    even = oracle.deinterlace_u8c3_f32c3(B.DEINTERLACE_INTER_LINEAR, 1, src)
+    assert np.all(even[0::2] == (2, 4, 8)) and np.all(even[1:7:2] == (2.5, 4.5, 8.5)) and np.all(even[7] == (1, 1, 1))
+    odd = oracle.deinterlace_u8c3_f32c3(B.DEINTERLACE_INTER_LINEAR, 0, src)
+    assert np.all(odd[1::2] == (1, 1, 1)) and np.all(odd[2::2] == (1.5, 1.5, 1.5)) and np.all(odd[0] == (2, 4, 8))
+    img = oracle.bytes(G.SEED, G.SRC)
+    for kind, ev in ((B.DEINTERLACE_BLEND, 1), (B.DEINTERLACE_INTER_LINEAR, 1), (B.DEINTERLACE_INTER_LINEAR, 0)):
+        assert same_bits(oracle.deinterlace_u8c3_f32c3(kind, ev, img), GOLD[f"deinterlace_{kind}_{ev}"])
+
+
+def test_deinterlace_closed_forms_and_reference(oracle, reference):
+    img = oracle.bytes(77, (12, 9, 3))
+    i32 = img.astype(np.int32)
+    blend = oracle.deinterlace_u8c3_f32c3(B.DEINTERLACE_BLEND, 1, img)
+    assert same_bits(blend[0], img[0].astype(np.float32)) and same_bits(blend[1:], ((i32[1:] + i32[:-1] + 1) * np.float32(0.5)).astype(np.float32))
+    even = oracle.deinterlace_u8c3_f32c3(B.DEINTERLACE_INTER_LINEAR, 1, img)
+    assert same_bits(even[0::2], img[0::2].astype(np.float32)) and same_bits(even[11], img[11].astype(np.float32))
+    assert same_bits(even[1:11:2], ((i32[0:10:2] + i32[2:12:2] + 1) * np.float32(0.5)).astype(np.float32))
+    odd_h = oracle.bytes(78, (7, 5, 3))  # an odd number of lines: the last line passes through in both fields
+    for ev in (0, 1):
+        assert same_bits(oracle.deinterlace_u8c3_f32c3(B.DEINTERLACE_INTER_LINEAR, ev, odd_h)[6], odd_h[6].astype(np.float32))
+    if reference.bw is not None:
+        for seed, shape in ((1, (2, 1, 3)), (2, (10, 33, 3)), (3, (64, 64, 3))):
+            a = oracle.bytes(seed, shape)
+            for kind, ev in ((B.DEINTERLACE_BLEND, 1), (B.DEINTERLACE_INTER_LINEAR, 1), (B.DEINTERLACE_INTER_LINEAR, 0)):
+                assert same_bits(oracle.deinterlace_u8c3_f32c3(kind, ev, a), reference.deinterlace_u8c3_f32c3(kind, ev, a))
