@@ -186,6 +186,35 @@ static_assert(std::is_same_v<std::decay_t<decltype(kBlend)>, ReadBack<Deinterlac
               std::is_same_v<std::decay_t<decltype(kRead.then(Deinterlace<DeinterlaceType::BLEND>::build()))>, std::decay_t<decltype(kBlend)>> &&
               std::is_same_v<std::decay_t<decltype(kBlend)>::Operation::OutputType, float3>);
 
+// SaturateCast over every pair of base types, at the lowest, half the highest and the highest input: the expectations
+// of the reference's utests/algorithm/image_processing/utest_saturate.h:46-85 (clamped to the output range, otherwise
+// the plain cast)
+template <typename I, typename O>
+constexpr bool saturate_pair_ok() {
+    constexpr I lowest = minValue<I>, half = maxValue<I> / 2, highest = maxValue<I>;
+    constexpr O want_low = cxp::cmp_less(lowest, minValue<O>) || !cxp::cmp_greater(lowest, minValue<O>) ? minValue<O> : static_cast<O>(lowest);
+    constexpr O want_half = cxp::cmp_greater(half, maxValue<O>) ? maxValue<O> : static_cast<O>(half);
+    constexpr O want_high = cxp::cmp_greater(highest, maxValue<O>) ? maxValue<O> : static_cast<O>(highest);
+    return SaturateCast<I, O>::exec(lowest) == want_low && SaturateCast<I, O>::exec(half) == want_half && SaturateCast<I, O>::exec(highest) == want_high &&
+           SaturateCast<VectorType_t<I, 3>, VectorType_t<O, 3>>::exec(make_set<VectorType_t<I, 3>>(highest)).z == want_high &&
+           SaturateCast<VectorType_t<I, 4>, VectorType_t<O, 4>>::exec(make_set<VectorType_t<I, 4>>(lowest)).w == want_low;
+}
+template <typename I, typename... Os>
+constexpr bool saturate_row_ok(TypeList<Os...>) {
+    return (saturate_pair_ok<I, Os>() && ...);
+}
+template <typename... Is>
+constexpr bool saturate_table_ok(TypeList<Is...> all) {
+    return (saturate_row_ok<Is>(all) && ...);
+}
+// integer -> float pairs are exact only while the integer fits the mantissa, so half / highest of 32-bit integers go
+// through the same cast on both sides and still compare equal
+static_assert(saturate_table_ok(TypeList<unsigned char, signed char, unsigned short, short, unsigned int, int, float, double>{}));
+static_assert(SaturateCast<float, uchar>::exec(254.5f) == 255 && SaturateCast<float, uchar>::exec(254.49f) == 254 && SaturateCast<float, uchar>::exec(0.5f) == 1 &&
+              SaturateCast<float, uchar>::exec(0.49999997f) == 1 && SaturateCast<float, uchar>::exec(0.4999999f) == 0 && SaturateCast<float, signed char>::exec(-0.5f) == -1 &&
+              SaturateCast<float, signed char>::exec(-128.7f) == -128 && SaturateCast<float, short>::exec(-2.5f) == -3 && SaturateCast<double, ushort>::exec(65534.5) == 65535,
+              "half away from zero through x + 0.5f (so the float just below one half rounds up, as in the reference), then the range");
+
 // DPP tags
 static_assert(TransformDPP<>::PAR_ARCH == ParArch::GPU_AMD && defaultParArch == ParArch::GPU_AMD && Stream::parArch() == ParArch::GPU_AMD);
 static_assert(exec::pixels_per_thread<float3, float3, false>() == 4 && exec::pixels_per_thread<uchar4, uchar, false>() == 4 &&
