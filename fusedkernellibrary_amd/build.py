@@ -88,6 +88,46 @@ def build_benchmarks():
     return out
 
 
+# The reference's own test headers that exercise this path's operator API (relative to the reference checkout); each
+# defines `int launch()`.  examples/readme_test_code.h is left out: half of it runs on the reference's CPU backend.
+REFERENCE_TESTS = (
+    "tests/algorithm/test_batchresize_build.h", "tests/algorithm/test_border_reader.h", "tests/algorithm/test_crop.h",
+    "tests/algorithm/test_deinterlace.h", "tests/algorithm/test_warp.h", "tests/data/test_ptr_nd.h", "tests/data/test_rect.h",
+    "tests/data/test_tuple.h", "tests/data/test_typelist.h", "tests/operation/test_filtered_index_sequence.h",
+    "tests/operation/test_fused_operation.h", "tests/operation/test_instantiable_operations.h",
+    "tests/operation/test_operation_fuser.h", "tests/operation/test_operation_tuple.h", "tests/operation/test_operation_types.h",
+    "tests/thread_fusion/test_thread_fusion.h",
+)
+REFERENCE_ROOT = os.environ.get("FK_REFERENCE_ROOT", "/root/reference")
+REFERENCE_TESTS_DIR = os.path.join(ROOT, "tests", "cpp", "reference_tests")
+
+
+def build_reference_tests():
+    """The reference's test headers compiled, unchanged and where they lie, against include/ of this library (their
+    #include <fused_kernel/...> lines resolve to the forwarding headers): most of their checks are static_asserts, so
+    compiling is already the larger part of the test; the programs run on the GPU box.  Nothing when no reference checkout
+    is present."""
+    if not os.path.isfile(os.path.join(REFERENCE_ROOT, REFERENCE_TESTS[0])):
+        return []
+    import tempfile
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(REFERENCE_TESTS_DIR, exist_ok=True)
+
+    def compile_one(header):
+        name = os.path.splitext(os.path.basename(header))[0]
+        out = os.path.join(REFERENCE_TESTS_DIR, name)
+        with tempfile.TemporaryDirectory() as tmp:
+            main = os.path.join(tmp, name + ".cpp")
+            with open(main, "w") as f:
+                f.write("#include <%s>\nint main() { return launch(); }\n" % header)
+            _run([hipcc(), "-x", "hip", main, "-I" + INCLUDE, "-I" + REFERENCE_ROOT, *DEVICE_FLAGS, "-L" + HERE, "-lfk_hip_rt",
+                  "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/../../../fusedkernellibrary_amd", "-o", out])
+        return out
+
+    with ThreadPoolExecutor(max_workers=4) as pool:
+        return list(pool.map(compile_one, REFERENCE_TESTS))
+
+
 def build_literal_capi():
     """The same chain entry points built with the reference's host-branch interpolation (bilinear row index taken from
     the x coordinate): only there to show parity with the reference CPU backend's own output where that is defined."""
@@ -99,7 +139,8 @@ def build_all():
     from concurrent.futures import ThreadPoolExecutor
     outs = [build_runtime()]  # the others link against it
     with ThreadPoolExecutor(max_workers=4) as pool:
-        jobs = [pool.submit(build_capi), pool.submit(build_literal_capi), pool.submit(build_cpp_tests), pool.submit(build_benchmarks)]
+        jobs = [pool.submit(build_capi), pool.submit(build_literal_capi), pool.submit(build_cpp_tests), pool.submit(build_benchmarks),
+                pool.submit(build_reference_tests)]
         for job in jobs:
             res = job.result()
             outs += res if isinstance(res, list) else [res]

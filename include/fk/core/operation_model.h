@@ -17,6 +17,7 @@
 #include <array>
 
 #include "fk/core/data.h"
+#include "fk/core/type_utils.h"
 
 namespace fk {
 
@@ -60,6 +61,14 @@ template <typename... Ts> constexpr bool notAllUnaryTypes = !allUnaryTypes<Ts...
 template <typename... Ts> constexpr bool noneWriteType = (!isWriteType<Ts> && ...);
 template <typename... Ts> constexpr bool noneMidWriteType = (!isMidWriteType<Ts> && ...);
 template <typename... Ts> constexpr bool noneAnyWriteType = (!isAnyWriteType<Ts> && ...);
+
+// A restriction for filtered_index_sequence_t over a list of kind tags: the kinds that carry parameters.
+struct NotUnaryRestriction {
+    template <typename Kind>
+    static constexpr bool complies() {
+        return !std::is_same_v<Kind, UnaryType>;
+    }
+};
 
 template <typename IOp> using GetInputType_t = typename IOp::Operation::InputType;
 template <typename IOp> using GetOutputType_t = typename IOp::Operation::OutputType;
@@ -227,6 +236,7 @@ struct OperationTuple<Operation_t, Rest...>
     static constexpr bool HAS_INSTANCE = !isUnaryType<Operation_t>;
     static constexpr bool HAS_NEXT = (sizeof...(Rest) > 0) && !allUnaryTypes<Rest...>;
     static constexpr bool HAS_REST = sizeof...(Rest) > 0;
+    using Next = OperationTuple<Rest...>; // the type list of the tail (a member `next` exists only where it holds data)
     enum { size = sizeof...(Rest) + 1 };
 };
 
@@ -275,6 +285,33 @@ FK_HD_CNST OperationTuple<As..., Bs...> operation_tuple_cat(const OperationTuple
     return out;
 }
 
+template <typename... As, typename... Bs>
+FK_HD_CNST OperationTuple<As..., Bs...> cat(const OperationTuple<As...>& a, const OperationTuple<Bs...>& b) {
+    return operation_tuple_cat(a, b);
+}
+
+namespace detail {
+template <typename Tuple_>
+FK_HD_CNST void tuple_assign(Tuple_&) {}
+template <typename Tuple_, typename First, typename... More>
+FK_HD_CNST void tuple_assign(Tuple_& t, const First& first, const More&... more) {
+    if constexpr (Tuple_::HAS_INSTANCE) {
+        t.instance = first;
+        if constexpr (sizeof...(More) > 0) tuple_assign(t.next, more...);
+    } else {
+        tuple_assign(t.next, first, more...);
+    }
+}
+} // namespace detail
+// An OperationTuple of the given operations, from the OperationData of those that have any (in order).
+template <typename... Operations, typename... Datas>
+FK_HD_CNST OperationTuple<Operations...> make_operation_tuple_(const Datas&... datas) {
+    static_assert(((isUnaryType<Operations> ? 0 : 1) + ...) == sizeof...(Datas), "One OperationData per operation that is not Unary.");
+    OperationTuple<Operations...> t{};
+    detail::tuple_assign(t, datas...);
+    return t;
+}
+
 // OperationData of element INDEX of the tuple; Unary elements have none.
 template <int INDEX, typename... Ops>
 FK_HD_CNST auto get(const OperationTuple<Ops...>& t) {
@@ -288,8 +325,6 @@ FK_HD_CNST auto get(const OperationTuple<Ops...>& t) {
 }
 
 namespace detail {
-template <int INDEX, typename Tuple>
-struct TupleElement;
 template <int INDEX, typename First, typename... Rest_>
 struct TupleElement<INDEX, OperationTuple<First, Rest_...>> {
     using type = typename TupleElement<INDEX - 1, OperationTuple<Rest_...>>::type;
@@ -298,45 +333,59 @@ template <typename First, typename... Rest_>
 struct TupleElement<0, OperationTuple<First, Rest_...>> {
     using type = First;
 };
+template <size_t N, typename... Ops>
+struct TypeAtImpl<N, OperationTuple<Ops...>> : TypeAtImpl<N, TypeList<Ops...>> {};
+template <int INDEX, typename TupleLike>
+struct ElementOf : TupleElement<INDEX, TupleLike> {};
+template <int INDEX, typename... Types>
+struct ElementOf<INDEX, TypeList<Types...>> : TypeAtImpl<static_cast<size_t>(INDEX), TypeList<Types...>> {};
 } // namespace detail
-template <int INDEX, typename Tuple>
-using get_type_t = typename detail::TupleElement<INDEX, Tuple>::type;
+template <int INDEX, typename TupleLike>
+using get_type_t = typename detail::ElementOf<INDEX, TupleLike>::type;
 
 // ---- FusedOperation -----------------------------------------------------------------------------------------
 namespace detail {
-// Runs the compute operations of a tuple in order on `input`.  The tuple is only ever walked by reference, so a
-// long chain stays in the registers (or kernel-argument scalars) it arrived in.
+// One operation of a fused chain applied to `input`: compute operations transform it; a write in the middle of a chain
+// stores it at `thread` and hands it on unchanged (a fused write-then-compute operation hands on its own result).
+template <typename Op, typename Input, typename Instance>
+FK_HD_CNST auto chain_step(const Point& thread, const Input& input, const Instance& holder) {
+    if constexpr (isUnaryType<Op>) {
+        return Op::exec(input);
+    } else if constexpr (isWriteType<Op>) {
+        Op::exec(thread, input, holder.instance);
+        return input;
+    } else if constexpr (isMidWriteType<Op>) {
+        return Op::exec(thread, input, holder.instance);
+    } else {
+        static_assert(isComputeType<Op>, "Only compute and write operations can follow the first operation of a fused chain.");
+        return Op::exec(input, holder.instance);
+    }
+}
+// Runs the operations of a tuple in order on `input`.  The tuple is only ever walked by reference, so a long chain
+// stays in the registers (or kernel-argument scalars) it arrived in.
 template <typename Input, typename Op, typename... Rest_>
-FK_HD_CNST auto tuple_compute(const Input& input, const OperationTuple<Op, Rest_...>& t) {
-    static_assert(isComputeType<Op>, "Only compute operations can follow the first operation of a fused chain.");
+FK_HD_CNST auto tuple_compute(const Point& thread, const Input& input, const OperationTuple<Op, Rest_...>& t) {
     using Tuple = OperationTuple<Op, Rest_...>;
     if constexpr (sizeof...(Rest_) == 0) {
-        if constexpr (isUnaryType<Op>) {
-            return Op::exec(input);
-        } else {
-            return Op::exec(input, t.instance);
-        }
+        return chain_step<Op>(thread, input, t);
     } else if constexpr (Tuple::HAS_NEXT) {
-        if constexpr (isUnaryType<Op>) {
-            return tuple_compute(Op::exec(input), t.next);
-        } else {
-            return tuple_compute(Op::exec(input, t.instance), t.next);
-        }
+        return tuple_compute(thread, chain_step<Op>(thread, input, t), t.next);
     } else { // the rest is Unary only and holds no data
-        if constexpr (isUnaryType<Op>) {
-            return tuple_compute(Op::exec(input), OperationTuple<Rest_...>{});
-        } else {
-            return tuple_compute(Op::exec(input, t.instance), OperationTuple<Rest_...>{});
-        }
+        return tuple_compute(thread, chain_step<Op>(thread, input, t), OperationTuple<Rest_...>{});
     }
+}
+template <typename Input, typename Op, typename... Rest_>
+FK_HD_CNST auto tuple_compute(const Input& input, const OperationTuple<Op, Rest_...>& t) {
+    static_assert(noneAnyWriteType<Op, Rest_...>, "A chain with writes needs the thread it runs for.");
+    return tuple_compute(Point(), input, t);
 }
 // Same, starting after the first element of the tuple (the read of a fused read chain).
 template <typename Input, typename Op, typename... Rest_>
-FK_HD_CNST auto tuple_compute_after_first(const Input& input, const OperationTuple<Op, Rest_...>& t) {
+FK_HD_CNST auto tuple_compute_after_first(const Point& thread, const Input& input, const OperationTuple<Op, Rest_...>& t) {
     if constexpr (OperationTuple<Op, Rest_...>::HAS_NEXT) {
-        return tuple_compute(input, t.next);
+        return tuple_compute(thread, input, t.next);
     } else {
-        return tuple_compute(input, OperationTuple<Rest_...>{});
+        return tuple_compute(thread, input, OperationTuple<Rest_...>{});
     }
 }
 template <typename... Ops>
@@ -353,6 +402,17 @@ template <typename Op, typename... Rest_>
 struct FirstOf {
     using type = Op;
 };
+// what a chain hands on after its last operation: that operation's output, or for a write the value it stored
+template <typename Op, typename = void>
+struct HandsOn {
+    using type = typename Op::OutputType;
+};
+template <typename Op>
+struct HandsOn<Op, std::enable_if_t<isWriteType<Op>>> {
+    using type = typename Op::InputType;
+};
+template <typename... Ops>
+using ChainOutput_t = typename HandsOn<typename LastOf<Ops...>::type>::type;
 } // namespace detail
 
 template <typename Enabler, typename... Operations>
@@ -372,7 +432,7 @@ public:
     using Operations = OperationTuple<FirstOp, ComputeOps...>;
     using ParamsType = OperationTuple<FirstOp, ComputeOps...>;
     using ReadDataType = typename FirstOp::ReadDataType;
-    using OutputType = typename detail::LastOf<FirstOp, ComputeOps...>::type::OutputType;
+    using OutputType = detail::ChainOutput_t<FirstOp, ComputeOps...>;
     using InstanceType = ReadType;
     using OperationDataType = OperationData<SelfType>;
     using InstantiableType = Read<SelfType>;
@@ -384,7 +444,7 @@ public:
         if constexpr (sizeof...(ComputeOps) == 0) {
             return FirstOp::exec(thread, params.instance);
         } else {
-            return detail::tuple_compute_after_first(FirstOp::exec(thread, params.instance), params);
+            return detail::tuple_compute_after_first(thread, FirstOp::exec(thread, params.instance), params);
         }
     }
     FK_HD_STATIC OutputType exec(const Point& thread, const OperationDataType& opData) { return exec(thread, opData.params); }
@@ -438,6 +498,34 @@ public:
     FK_HD_STATIC InstantiableType build(const OperationDataType& opData) { return InstantiableType{ opData }; }
 };
 
+// A chain that starts with a write: stores its input at the thread's position, runs the rest on it and hands the result
+// on, so as a whole it behaves as one MidWrite operation.
+template <typename FirstOp, typename... Ops>
+struct FusedOperation_<std::enable_if_t<isAnyWriteType<FirstOp>>, FirstOp, Ops...> {
+private:
+    using SelfType = FusedOperation_<void, FirstOp, Ops...>;
+
+public:
+    FK_STATIC_STRUCT(FusedOperation_, SelfType)
+    using ParamsType = OperationTuple<FirstOp, Ops...>;
+    using InputType = typename FirstOp::InputType;
+    using OutputType = detail::ChainOutput_t<FirstOp, Ops...>;
+    using WriteDataType = typename FirstOp::WriteDataType;
+    using InstanceType = MidWriteType;
+    using OperationDataType = OperationData<SelfType>;
+    using InstantiableType = MidWrite<SelfType>;
+    static constexpr bool IS_FUSED_OP = true;
+    static constexpr bool THREAD_FUSION = false;
+    FK_HD_STATIC OutputType exec(const Point& thread, const InputType& input, const ParamsType& params) {
+        return detail::tuple_compute(thread, input, params);
+    }
+    FK_HD_STATIC OutputType exec(const Point& thread, const InputType& input, const OperationDataType& opData) {
+        return exec(thread, input, opData.params);
+    }
+    FK_HD_STATIC InstantiableType build(const ParamsType& params) { return InstantiableType{ { params } }; }
+    FK_HD_STATIC InstantiableType build(const OperationDataType& opData) { return InstantiableType{ opData }; }
+};
+
 namespace detail {
 // One IOp as an OperationTuple: fused IOps contribute their whole tuple, so chains never nest.
 template <typename IOp>
@@ -467,6 +555,39 @@ FK_HD_CNST auto tuple_to_iop(const OperationTuple<Ops...>& t) {
     }
 }
 } // namespace detail
+
+// The OperationTuple of a sequence of IOps; fused IOps contribute their elements.
+template <typename IOp>
+FK_HD_CNST auto iOpsToOperationTuple(const IOp& iOp) {
+    return detail::iop_to_tuple(iOp);
+}
+template <typename IOp, typename... IOps>
+FK_HD_CNST auto iOpsToOperationTuple(const IOp& iOp, const IOps&... iOps) {
+    return operation_tuple_cat(detail::iop_to_tuple(iOp), iOpsToOperationTuple(iOps...));
+}
+
+// An all-Unary FusedOperation carries its operations as a type only; any other one as a tuple of their data.
+template <typename Operation, typename = void>
+struct IsAllUnaryFusedOperation : std::false_type {};
+template <typename Operation>
+struct IsAllUnaryFusedOperation<Operation, std::enable_if_t<detail::IsFused<Operation>::value && isUnaryType<Operation>>> : std::true_type {};
+template <typename Operation>
+constexpr bool isAllUnaryFusedOperation = IsAllUnaryFusedOperation<Operation>::value;
+template <typename Operation>
+constexpr bool isNotAllUnaryFusedOperation = !isAllUnaryFusedOperation<Operation>;
+
+// Both directions between a fused IOp and the OperationTuple it stands for.
+template <typename FusedIOp>
+struct InstantiableFusedOperationToOperationTuple {
+    static_assert(detail::IsFused<typename FusedIOp::Operation>::value, "Not a fused operation.");
+    FK_HD_STATIC auto value(const FusedIOp& iOp) { return detail::iop_to_tuple(iOp); }
+};
+template <typename Tuple_>
+struct OperationTupleToInstantiableOperation;
+template <typename... Operations>
+struct OperationTupleToInstantiableOperation<OperationTuple<Operations...>> {
+    FK_HD_STATIC auto value(const OperationTuple<Operations...>& t) { return detail::tuple_to_iop(t); }
+};
 
 // ---- batch reads ----------------------------------------------------------------------------------------------
 enum class PlanePolicy { PROCESS_ALL = 0, CONDITIONAL_WITH_DEFAULT = 1 };
@@ -635,6 +756,53 @@ struct BatchBuilders {
             return BatchRead<BATCH_N, PlanePolicy::CONDITIONAL_WITH_DEFAULT>::build(
                 BatchOperation::build_batch<Self>(first, arrays...), usedPlanes, defaultValue);
         }
+    }
+};
+
+// ---- batch writes ---------------------------------------------------------------------------------------------
+// BATCH writes of one kind behind one Write operation: plane thread.z goes to its own destination
+// (operation_model/batch_operations.h:320-377).  The parameters are the plain array of the per-plane parameters.
+template <size_t BATCH_, typename Operation_ = void>
+struct BatchWrite {
+private:
+    using SelfType = BatchWrite<BATCH_, Operation_>;
+
+public:
+    FK_STATIC_STRUCT(BatchWrite, SelfType)
+    static_assert(isWriteType<Operation_>, "The Operation is not of Write type");
+    using Operation = Operation_;
+    static constexpr size_t BATCH = BATCH_;
+    using InputType = typename Operation::InputType;
+    using ParamsType = typename Operation::ParamsType[BATCH_];
+    using WriteDataType = typename Operation::WriteDataType;
+    using InstanceType = WriteType;
+    using OperationDataType = OperationData<SelfType>;
+    using InstantiableType = Write<SelfType>;
+    static constexpr bool IS_FUSED_OP = false;
+    static constexpr bool THREAD_FUSION = false;
+
+    FK_HD_STATIC void exec(const Point& thread, const InputType& input, const ParamsType& params) { Operation::exec(thread, input, params[thread.z]); }
+    FK_HD_STATIC void exec(const Point& thread, const InputType& input, const OperationDataType& opData) { exec(thread, input, opData.params); }
+    FK_HD_STATIC uint num_elems_x(const Point& thread, const OperationDataType& opData) { return Operation::num_elems_x(thread, { opData.params[thread.z] }); }
+    FK_HD_STATIC uint pitch(const Point& thread, const OperationDataType& opData) { return Operation::pitch(thread, { opData.params[thread.z] }); }
+    template <typename IOp>
+    static inline constexpr std::enable_if_t<isWriteType<IOp>, InstantiableType> build(const std::array<IOp, BATCH_>& iOps) {
+        static_assert(std::is_same_v<typename IOp::Operation, Operation_>, "The IOps in the array are of another operation");
+        InstantiableType out{};
+        for (size_t i = 0; i < BATCH_; ++i) out.params[i] = iOps[i].params;
+        return out;
+    }
+    template <typename First, typename... Arrays>
+    static inline constexpr std::enable_if_t<!isWriteType<First>, InstantiableType> build(const std::array<First, BATCH_>& first, const Arrays&... arrays) {
+        return build(Operation::build_batch(first, arrays...));
+    }
+};
+// Builder form: BatchWrite<N>::build(array of Write IOps).
+template <size_t BATCH_>
+struct BatchWrite<BATCH_, void> {
+    template <typename IOp>
+    static inline constexpr auto build(const std::array<IOp, BATCH_>& iOps) {
+        return BatchWrite<BATCH_, typename IOp::Operation>::build(iOps);
     }
 };
 

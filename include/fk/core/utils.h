@@ -46,7 +46,9 @@ using ulonglong = unsigned long long;
 struct NullType {};
 
 template <typename... Types>
-struct TypeList {};
+struct TypeList {
+    enum { size = sizeof...(Types) };
+};
 
 // Throws std::runtime_error("GPU Error: <text> File: <file> Line: <line>") on a non-zero runtime status, the
 // text convention of the reference's gpuAssert (core/utils/utils.h:95-109).

@@ -18,7 +18,26 @@ namespace fk {
     struct NAME##3 { BASE x, y, z; };                                                                                  \
     struct alignas(A4) NAME##4 { BASE x, y, z, w; };
 
-FK_DEFINE_VECTOR_FAMILY(bool, bool, 2, 4)
+// Vectors of bool (the result of comparing two vectors) also convert to one bool: true when every channel is.
+struct bool1 { bool x; __host__ __device__ constexpr operator bool() const { return x; } };
+struct bool2 { bool x, y; __host__ __device__ constexpr operator bool() const { return x && y; } };
+struct bool3 { bool x, y, z; __host__ __device__ constexpr operator bool() const { return x && y && z; } };
+struct bool4 { bool x, y, z, w; __host__ __device__ constexpr operator bool() const { return x && y && z && w; } };
+using Bool1 = bool1;
+using Bool2 = bool2;
+using Bool3 = bool3;
+using Bool4 = bool4;
+// All / any channel of a bool vector.
+struct Bool {
+    static constexpr __host__ __device__ bool vAnd(const bool1& v) { return v.x; }
+    static constexpr __host__ __device__ bool vAnd(const bool2& v) { return v.x && v.y; }
+    static constexpr __host__ __device__ bool vAnd(const bool3& v) { return v.x && v.y && v.z; }
+    static constexpr __host__ __device__ bool vAnd(const bool4& v) { return v.x && v.y && v.z && v.w; }
+    static constexpr __host__ __device__ bool vOr(const bool1& v) { return v.x; }
+    static constexpr __host__ __device__ bool vOr(const bool2& v) { return v.x || v.y; }
+    static constexpr __host__ __device__ bool vOr(const bool3& v) { return v.x || v.y || v.z; }
+    static constexpr __host__ __device__ bool vOr(const bool4& v) { return v.x || v.y || v.z || v.w; }
+};
 FK_DEFINE_VECTOR_FAMILY(char, signed char, 2, 4)
 FK_DEFINE_VECTOR_FAMILY(uchar, unsigned char, 2, 4)
 FK_DEFINE_VECTOR_FAMILY(short, short, 4, 8)
@@ -126,7 +145,7 @@ FK_HD_CNST VBase<T> vectorAt(int idx, const T& v) {
 template <typename T, typename... Numbers>
 FK_HD_CNST T make_(const Numbers&... pack) {
     if constexpr (validCUDAVec<T>) {
-        static_assert(sizeof...(Numbers) == cn<T>, "make_: one argument per channel");
+        static_assert(sizeof...(Numbers) <= cn<T>, "make_: at most one argument per channel (channels left out are zero)");
         return T{ static_cast<VBase<T>>(pack)... };
     } else {
         static_assert(sizeof...(Numbers) == 1, "make_: a scalar takes one argument");

@@ -719,7 +719,7 @@ struct ResizeJob {
 // ---- generic -----------------------------------------------------------------------------------------------------
 template <typename Sender, typename Receiver>
 struct GenericJob {
-    static constexpr bool READ_IN_PLACE = isBatchOperation<typename Sender::Operation>;
+    static constexpr bool READ_IN_PLACE = isBatchOperation<typename Sender::Operation> || isBatchOperation<typename Receiver::Operation>;
     Sender sender;
     Receiver receiver;
     ActiveThreads active;

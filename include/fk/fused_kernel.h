@@ -3,6 +3,7 @@
 #ifndef FK_FUSED_KERNEL_H
 #define FK_FUSED_KERNEL_H
 
+#include "fk/core/thread_fusion_info.h"
 #include "fk/exec/executor.h"
 #include "fk/ops/yuv.h"
 #include "fk/ops/border_reader.h"

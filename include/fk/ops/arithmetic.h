@@ -7,6 +7,7 @@
 
 #include <limits>
 
+#include "fk/core/constexpr_cmath.h"
 #include "fk/core/operation_model.h"
 
 namespace fk {
@@ -45,11 +46,33 @@ namespace fk {
             return detail::cast_channels<O>(input OP params);                                                          \
         }                                                                                                              \
     };
-FK_ARITHMETIC_OPERATION(Add, +)
 FK_ARITHMETIC_OPERATION(Sub, -)
 FK_ARITHMETIC_OPERATION(Mul, *)
 FK_ARITHMETIC_OPERATION(Div, /)
 #undef FK_ARITHMETIC_OPERATION
+
+// Add has two forms: Binary (input + parameter), and Unary over a Tuple of both operands (basic_ops/arithmetic.h:21-48).
+template <typename I1, typename I2 = I1, typename O = I1, typename IT = BinaryType>
+struct Add;
+template <typename I, typename P, typename O>
+struct Add<I, P, O, BinaryType> {
+private:
+    using SelfType = Add<I, P, O, BinaryType>;
+
+public:
+    FK_BINARY_OPERATION(Add, I, P, O)
+    FK_HD_STATIC OutputType exec(const InputType& input, const ParamsType& params) { return detail::cast_channels<O>(input + params); }
+};
+template <typename I1, typename I2, typename O>
+struct Add<I1, I2, O, UnaryType> {
+private:
+    using SelfType = Add<I1, I2, O, UnaryType>;
+    using Operands = Tuple<I1, I2>;
+
+public:
+    FK_UNARY_OPERATION(Add, Operands, O)
+    FK_HD_STATIC OutputType exec(const InputType& input) { return detail::cast_channels<O>(get<0>(input) + get<1>(input)); }
+};
 
 // static_cast per channel
 template <typename I, typename O>
@@ -63,34 +86,6 @@ public:
     FK_HD_STATIC OutputType exec(const InputType& input) { return detail::cast_channels<O>(input); }
 };
 
-namespace cxp {
-// Half away from zero through an int cast (constexpr_cmath.h:119-130).
-template <typename T>
-FK_HD_CNST T round(T x) {
-    static_assert(std::is_floating_point_v<T>, "Input must be a floating-point type");
-    if (x != x || x == std::numeric_limits<T>::infinity() || x == -std::numeric_limits<T>::infinity()) return x;
-    return (x > T(0)) ? static_cast<T>(static_cast<int>(x + T(0.5))) : static_cast<T>(static_cast<int>(x - T(0.5)));
-}
-template <typename T>
-FK_HD_CNST T max(const T& a, const T& b) { return a >= b ? a : b; }
-template <typename T>
-FK_HD_CNST T min(const T& a, const T& b) { return a <= b ? a : b; }
-// Sign-safe comparisons between arithmetic types (constexpr_cmath.h:75-117).
-template <typename T, typename U>
-FK_HD_CNST bool cmp_less(const T& t, const U& u) {
-    if constexpr (std::is_floating_point_v<T> || std::is_floating_point_v<U>) {
-        return t < u;
-    } else if constexpr (std::is_signed_v<T> == std::is_signed_v<U>) {
-        return t < u;
-    } else if constexpr (std::is_signed_v<T>) {
-        return t < 0 || static_cast<std::make_unsigned_t<T>>(t) < u;
-    } else {
-        return u >= 0 && t < static_cast<std::make_unsigned_t<U>>(u);
-    }
-}
-template <typename T, typename U>
-FK_HD_CNST bool cmp_greater(const T& t, const U& u) { return cmp_less(u, t); }
-} // namespace cxp
 
 template <typename T>
 constexpr T maxValue = std::numeric_limits<T>::max();
@@ -182,23 +177,237 @@ public:
     FK_HD_STATIC OutputType exec(const InputType& input) { return detail::cast_channels<O>(input); }
 };
 
-template <typename I, typename P = I, typename O = I>
-struct Max {
+// ---- per-channel application of a scalar operation (operation_model/vector_operations.h:23-189) -----------------
+// UnaryV<Op, I, O>: O{ Op(i.x), Op(i.y), ... }; with a Tuple<I1, I2> input Op gets Tuple{ i1.x, i2.x } per channel, where
+// a scalar second operand is used for every channel.  BinaryV<Op, I, P, O>: O{ Op(i.x, p.x), ... }, same rule for P.
+namespace detail {
+template <typename In, typename Out>
+constexpr bool both_vectors_or_none = validCUDAVec<In> == validCUDAVec<Out>;
+}
+template <typename Operation, typename I, typename O, typename = void>
+struct UnaryV {
 private:
-    using SelfType = Max<I, P, O>;
+    using SelfType = UnaryV<Operation, I, O, void>;
+    template <int... K>
+    FK_HD_STATIC O channels(const I& input, std::integer_sequence<int, K...>) {
+        if constexpr (validCUDAVec<O>) {
+            return O{ Operation::exec(vget<K>(input))... };
+        } else {
+            return Operation::exec(input);
+        }
+    }
 
 public:
-    FK_BINARY_OPERATION(Max, I, P, O)
-    FK_HD_STATIC OutputType exec(const InputType& input, const ParamsType& params) { return static_cast<O>(input >= params ? input : params); }
+    FK_STATIC_STRUCT(UnaryV, SelfType)
+    using InputType = I;
+    using OutputType = O;
+    using InstanceType = UnaryType;
+    static_assert(cn<I> == cn<O>, "UnaryV requires the same number of channels for input and output types.");
+    static_assert(detail::both_vectors_or_none<I, O>, "UnaryV requires input and output types to be both vector types or none.");
+    FK_HD_STATIC OutputType exec(const InputType& input) { return channels(input, std::make_integer_sequence<int, cn<I>>{}); }
 };
-template <typename I, typename P = I, typename O = I>
-struct Min {
+template <typename Operation, typename I, typename O>
+struct UnaryV<Operation, I, O, std::enable_if_t<isTuple_v<I>>> {
 private:
-    using SelfType = Min<I, P, O>;
+    using SelfType = UnaryV<Operation, I, O, void>;
+    using I1 = get_t<0, I>;
+    using I2 = get_t<1, I>;
+    template <int... K>
+    FK_HD_STATIC O channels(const I1& a, const I2& b, std::integer_sequence<int, K...>) {
+        using Pair = typename Operation::InputType;
+        if constexpr (validCUDAVec<O>) {
+            return O{ Operation::exec(Pair{ vget<K>(a), vget<K>(b) })... };
+        } else {
+            return Operation::exec(Pair{ a, b });
+        }
+    }
 
 public:
-    FK_BINARY_OPERATION(Min, I, P, O)
-    FK_HD_STATIC OutputType exec(const InputType& input, const ParamsType& params) { return static_cast<O>(input <= params ? input : params); }
+    FK_STATIC_STRUCT(UnaryV, SelfType)
+    using InputType = I;
+    using OutputType = O;
+    using InstanceType = UnaryType;
+    static_assert(cn<I1> == cn<O>, "UnaryV requires the same number of channels for input and output types.");
+    static_assert(detail::both_vectors_or_none<I1, O>, "UnaryV requires input and output types to be both vector types or none.");
+    FK_HD_STATIC OutputType exec(const InputType& input) { return channels(get<0>(input), get<1>(input), std::make_integer_sequence<int, cn<I1>>{}); }
+};
+template <typename Operation, typename I, typename P = I, typename O = I>
+struct BinaryV {
+private:
+    using SelfType = BinaryV<Operation, I, P, O>;
+    template <int... K>
+    FK_HD_STATIC O channels(const I& input, const P& params, std::integer_sequence<int, K...>) {
+        if constexpr (validCUDAVec<O>) {
+            return O{ Operation::exec(vget<K>(input), vget<K>(params))... };
+        } else {
+            return Operation::exec(input, params);
+        }
+    }
+
+public:
+    FK_STATIC_STRUCT(BinaryV, SelfType)
+    using InputType = I;
+    using ParamsType = P;
+    using OutputType = O;
+    using InstanceType = BinaryType;
+    using OperationDataType = OperationData<SelfType>;
+    static_assert(cn<I> == cn<O>, "BinaryV requires the same number of channels for input and output types.");
+    static_assert(detail::both_vectors_or_none<I, O>, "BinaryV requires input and output types to be both vector types or none.");
+    FK_HD_STATIC OutputType exec(const InputType& input, const ParamsType& params) { return channels(input, params, std::make_integer_sequence<int, cn<I>>{}); }
+    FK_HD_STATIC OutputType exec(const InputType& input, const OperationDataType& opData) { return exec(input, opData.params); }
+};
+
+// ---- Max / Min (basic_ops/logical.h:84-194): per channel, on a tie the parameter; Binary and Tuple-input Unary forms --
+#define FK_EXTREME_OPERATION(NAME, BASE, PICK)                                                                         \
+    template <typename I, typename P = I, typename O = I, typename IT = BinaryType>                                    \
+    struct BASE {                                                                                                      \
+    private:                                                                                                           \
+        using SelfType = BASE<I, P, O, BinaryType>;                                                                    \
+                                                                                                                       \
+    public:                                                                                                            \
+        FK_BINARY_OPERATION(BASE, I, P, O)                                                                             \
+        static_assert(!validCUDAVec<I> && !validCUDAVec<P> && !validCUDAVec<O>, #BASE " works on scalars.");           \
+        FK_HD_STATIC OutputType exec(const InputType& input, const ParamsType& params) { return cxp::PICK(input, params); } \
+    };                                                                                                                 \
+    template <typename I, typename P, typename O>                                                                      \
+    struct BASE<I, P, O, UnaryType> {                                                                                  \
+    private:                                                                                                           \
+        using SelfType = BASE<I, P, O, UnaryType>;                                                                     \
+        using Operands = Tuple<I, P>;                                                                                  \
+                                                                                                                       \
+    public:                                                                                                            \
+        FK_UNARY_OPERATION(BASE, Operands, O)                                                                          \
+        static_assert(!validCUDAVec<I> && !validCUDAVec<P> && !validCUDAVec<O>, #BASE " works on scalars.");           \
+        FK_HD_STATIC OutputType exec(const InputType& input) { return cxp::PICK(get<0>(input), get<1>(input)); }       \
+    };                                                                                                                 \
+    template <typename I, typename P = I, typename O = I, typename IT = BinaryType>                                    \
+    struct NAME {                                                                                                      \
+    private:                                                                                                           \
+        using SelfType = NAME<I, P, O, BinaryType>;                                                                    \
+                                                                                                                       \
+    public:                                                                                                            \
+        FK_BINARY_OPERATION(NAME, I, P, O)                                                                             \
+        FK_HD_STATIC OutputType exec(const InputType& input, const ParamsType& params) {                               \
+            return BinaryV<BASE<VBase<I>, VBase<P>, VBase<O>>, I, P, O>::exec(input, params);                          \
+        }                                                                                                              \
+    };                                                                                                                 \
+    template <typename I, typename P, typename O>                                                                      \
+    struct NAME<I, P, O, UnaryType> {                                                                                  \
+    private:                                                                                                           \
+        using SelfType = NAME<I, P, O, UnaryType>;                                                                     \
+        using Operands = Tuple<I, P>;                                                                                  \
+                                                                                                                       \
+    public:                                                                                                            \
+        FK_UNARY_OPERATION(NAME, Operands, O)                                                                          \
+        FK_HD_STATIC OutputType exec(const InputType& input) {                                                         \
+            return UnaryV<BASE<VBase<I>, VBase<P>, VBase<O>, UnaryType>, Operands, O>::exec(input);                    \
+        }                                                                                                              \
+    };
+FK_EXTREME_OPERATION(Max, MaxBase, max)
+FK_EXTREME_OPERATION(Min, MinBase, min)
+#undef FK_EXTREME_OPERATION
+
+// All channels of both operands equal (basic_ops/logical.h:196-223).
+template <typename I1, typename I2 = I1>
+struct Equal {
+private:
+    using SelfType = Equal<I1, I2>;
+    using Operands = Tuple<I1, I2>;
+
+public:
+    FK_UNARY_OPERATION(Equal, Operands, bool)
+    FK_HD_STATIC OutputType exec(const InputType& input) {
+        if constexpr (validCUDAVec<I1>) {
+            return Bool::vAnd(get<0>(input) == get<1>(input));
+        } else {
+            return get<0>(input) == get<1>(input);
+        }
+    }
+};
+
+// ---- more vector operations (basic_ops/cuda_vector.h:75-176) ---------------------------------------------------------
+// Channel permutation chosen at run time: output channel k takes input channel params[k].
+template <typename T>
+struct VectorReorderRT {
+private:
+    using SelfType = VectorReorderRT<T>;
+    using Order = VectorType_t<int, cn<T>>;
+    template <int... K>
+    FK_HD_STATIC T pick(const T& input, const Order& order, std::integer_sequence<int, K...>) {
+        const VBase<T> channel[cn<T>]{ vget<K>(input)... };
+        return T{ channel[vget<K>(order)]... };
+    }
+
+public:
+    FK_BINARY_OPERATION(VectorReorderRT, T, Order, T)
+    static_assert(validCUDAVec<T> && cn<T> >= 2, "VectorReorderRT needs a vector type with two or more channels");
+    FK_HD_STATIC OutputType exec(const InputType& input, const ParamsType& params) { return pick(input, params, std::make_integer_sequence<int, cn<T>>{}); }
+};
+
+// Folds the channels from left to right with a two-operand operation: Op(Op(x, y), z)...  The operation is Binary, or Unary
+// over a Tuple of both operands.
+template <typename T, typename Operation>
+struct VectorReduce {
+private:
+    using SelfType = VectorReduce<T, Operation>;
+    using Result = typename Operation::OutputType;
+    template <typename A, typename B>
+    FK_HD_STATIC Result combine(const A& a, const B& b) {
+        if constexpr (isUnaryType<Operation>) {
+            using Pair = typename Operation::InputType;
+            return Operation::exec(Pair{ static_cast<get_t<0, Pair>>(a), static_cast<get_t<1, Pair>>(b) });
+        } else {
+            return Operation::exec(a, b);
+        }
+    }
+
+public:
+    FK_UNARY_OPERATION(VectorReduce, T, Result)
+    FK_HD_STATIC OutputType exec(const InputType& input) {
+        if constexpr (cn<T> == 1) {
+            return vget<0>(input);
+        } else if constexpr (cn<T> == 2) {
+            return combine(input.x, input.y);
+        } else if constexpr (cn<T> == 3) {
+            return combine(combine(input.x, input.y), input.z);
+        } else {
+            return combine(combine(combine(input.x, input.y), input.z), input.w);
+        }
+    }
+};
+
+// The channels of a bool vector folded with equality, as the reference defines it (cuda_vector.h:157-169): true for an
+// all-true vector, and the fold (x == y) == z ... for any other.
+template <typename T>
+struct VectorAnd {
+private:
+    using SelfType = VectorAnd<T>;
+
+public:
+    FK_UNARY_OPERATION(VectorAnd, T, bool)
+    FK_HD_STATIC OutputType exec(const InputType& input) { return VectorReduce<T, Equal<bool, bool>>::exec(input); }
+};
+template <typename T>
+FK_HD_CNST bool vecAnd(const T& value) {
+    return VectorAnd<T>::exec(value);
+}
+
+// Appends the parameter as one more channel.
+template <typename I, typename O>
+struct AddLast {
+private:
+    using SelfType = AddLast<I, O>;
+    using Channel = VBase<I>;
+    template <int... K>
+    FK_HD_STATIC O append(const I& input, const Channel& last, std::integer_sequence<int, K...>) {
+        return O{ vget<K>(input)..., last };
+    }
+
+public:
+    FK_BINARY_OPERATION(AddLast, I, Channel, O)
+    static_assert(cn<I> == cn<O> - 1, "Output type should have one channel more");
+    static_assert(std::is_same_v<VBase<I>, VBase<O>>, "Base types should be the same");
+    FK_HD_STATIC OutputType exec(const InputType& input, const ParamsType& params) { return append(input, params, std::make_integer_sequence<int, cn<I>>{}); }
 };
 
 } // namespace fk

@@ -81,10 +81,15 @@ public:
     FK_HD_STATIC uint pitch(const Point&, const OperationDataType& opData) { return opData.params.dims.pitch; }
     // one write per buffer (memory_operations.h:113-152: the batch builders of a write return the array itself)
     template <size_t BATCH_N, typename Buffer>
-    static inline std::array<InstantiableType, BATCH_N> build_batch(const std::array<Buffer, BATCH_N>& buffers) {
+    static inline constexpr std::array<InstantiableType, BATCH_N> build_batch(const std::array<Buffer, BATCH_N>& buffers) {
         std::array<InstantiableType, BATCH_N> out{};
         for (size_t i = 0; i < BATCH_N; ++i) out[i] = build(buffers[i]);
         return out;
+    }
+    // all of them behind one Write operation: plane z of the launch goes to buffer z
+    template <size_t BATCH_N, typename Buffer>
+    static inline constexpr auto build(const std::array<Buffer, BATCH_N>& buffers) {
+        return BatchWrite<BATCH_N, SelfType>::build(build_batch(buffers));
     }
     FK_HD_STATIC InstantiableType build(const ParamsType& params) { return InstantiableType{ { params } }; }
     FK_HD_STATIC InstantiableType build(const OperationDataType& opData) { return InstantiableType{ opData }; }
