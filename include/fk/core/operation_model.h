@@ -55,6 +55,15 @@ template <typename T> constexpr bool isTernaryType = detail::is_kind<T, TernaryT
 template <typename T> constexpr bool isWriteType = detail::is_kind<T, WriteType>;
 template <typename T> constexpr bool isMidWriteType = detail::is_kind<T, MidWriteType>;
 template <typename T> constexpr bool isAnyWriteType = isWriteType<T> || isMidWriteType<T>;
+// the same as class templates, for use in template argument lists
+template <typename T> struct IsReadType : std::bool_constant<isReadType<T>> {};
+template <typename T> struct IsReadBackType : std::bool_constant<isReadBackType<T>> {};
+template <typename T> struct IsUnaryType : std::bool_constant<isUnaryType<T>> {};
+template <typename T> struct IsBinaryType : std::bool_constant<isBinaryType<T>> {};
+template <typename T> struct IsTernaryType : std::bool_constant<isTernaryType<T>> {};
+template <typename T> struct IsMidWriteType : std::bool_constant<isMidWriteType<T>> {};
+template <typename T> struct IsWriteType : std::bool_constant<isWriteType<T>> {};
+using WriteTypeList = TypeList<WriteType, MidWriteType>;
 template <typename T> constexpr bool isComputeType = isUnaryType<T> || isBinaryType<T> || isTernaryType<T>;
 template <typename... Ts> constexpr bool allUnaryTypes = (isUnaryType<Ts> && ...);
 template <typename... Ts> constexpr bool notAllUnaryTypes = !allUnaryTypes<Ts...>;

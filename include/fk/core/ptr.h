@@ -146,6 +146,20 @@ public:
     ~Ptr() { release(); }
 
     Ptr(const PtrDims<D>& dims, const MemType& type_ = defaultMemType, const int& deviceID_ = 0) { allocPtr(dims, type_, deviceID_); }
+    // Allocation by extent, one form per dimensionality (core/data/ptr_nd.h:303-320).
+    template <ND DN = D, std::enable_if_t<DN == ND::_1D, int> = 0>
+    Ptr(const uint& num_elems, const uint& size_in_bytes = 0, const MemType& type_ = defaultMemType, const int& deviceID_ = 0) {
+        allocPtr(PtrDims<ND::_1D>(num_elems, size_in_bytes), type_, deviceID_);
+    }
+    template <ND DN = D, std::enable_if_t<DN == ND::_2D, int> = 0>
+    Ptr(const uint& width_, const uint& height_, const uint& pitch_ = 0, const MemType& type_ = defaultMemType, const int& deviceID_ = 0) {
+        allocPtr(PtrDims<ND::_2D>(width_, height_, pitch_), type_, deviceID_);
+    }
+    template <ND DN = D, std::enable_if_t<DN == ND::_3D, int> = 0>
+    Ptr(const uint& width_, const uint& height_, const uint& planes_, const uint& color_planes_ = 1, const uint& pitch_ = 0,
+        const MemType& type_ = defaultMemType, const int& deviceID_ = 0) {
+        allocPtr(PtrDims<ND::_3D>(width_, height_, planes_, color_planes_, pitch_), type_, deviceID_);
+    }
 
     // Non-owning views over memory the caller manages.
     Ptr(T* data_, const PtrDims<D>& dims, const MemType& type_, const int& deviceID_) {

@@ -83,7 +83,7 @@ private:
 template <bool THREAD_FUSION_ENABLED, typename... IOpTypes>
 FK_HD_CNST bool isThreadFusionEnabled() {
     using ReadOperation = typename TypeAt_t<0, TypeList<IOpTypes...>>::Operation;
-    using WriteOperation = typename TypeAt_t<sizeof...(IOpTypes) - 1, TypeList<IOpTypes...>>::Operation;
+    using WriteOperation = typename TypeAt_t<-1, TypeList<IOpTypes...>>::Operation;
     return ReadOperation::THREAD_FUSION && WriteOperation::THREAD_FUSION && THREAD_FUSION_ENABLED;
 }
 } // namespace fk

@@ -64,8 +64,9 @@ template <typename T, typename First, typename... Rest>
 struct IndexOf<T, TypeList<First, Rest...>> : std::integral_constant<size_t, 1 + IndexOf<T, TypeList<Rest...>>::value> {};
 } // namespace detail
 
-template <size_t N, typename List>
-using TypeAt_t = typename detail::TypeAtImpl<N, List>::type;
+// element N of a list; -1 names the last one
+template <int N, typename List>
+using TypeAt_t = typename detail::TypeAtImpl<(N < 0 ? static_cast<size_t>(List::size) - 1 : static_cast<size_t>(N)), List>::type;
 template <typename... Lists>
 using TypeListCat_t = typename detail::TypeListCatImpl<Lists...>::type;
 template <typename List, typename T>
@@ -84,7 +85,82 @@ template <typename T, typename List>
 constexpr size_t TypeIndex_v = detail::IndexOf<T, List>::value;
 // the type of ListTwo at the place T has in ListOne
 template <typename T, typename ListOne, typename ListTwo>
-using EquivalentType_t = TypeAt_t<TypeIndex_v<T, ListOne>, ListTwo>;
+using EquivalentType_t = TypeAt_t<static_cast<int>(TypeIndex_v<T, ListOne>), ListTwo>;
+// the list without element N
+template <size_t N, typename List>
+using RemoveType_t = TypeListCat_t<typename detail::SplitAt<N, TypeList<>, List>::head,
+                                   typename detail::SplitAt<1, TypeList<>, typename detail::SplitAt<N, TypeList<>, List>::tail>::tail>;
+template <typename T, typename List>
+constexpr bool all_of_v = false;
+template <typename T, typename... Ts>
+constexpr bool all_of_v<T, TypeList<Ts...>> = (std::is_same_v<T, Ts> && ...);
+// the same queries as class templates
+template <typename T>
+struct IsTypeList : std::bool_constant<isTypeList<T>> {};
+template <typename T, typename List>
+struct one_of : std::bool_constant<one_of_v<T, List>> {};
+template <typename T, typename List>
+struct all_of : std::bool_constant<all_of_v<T, List>> {};
+template <typename T, typename List>
+struct TypeIndex : std::integral_constant<size_t, TypeIndex_v<T, List>> {};
+template <typename ListOne, typename ListTwo>
+struct TypeListCat {
+    using type = TypeListCat_t<ListOne, ListTwo>;
+};
+// an enumerator as a type
+template <typename Enum, Enum VALUE>
+struct EnumType {};
+template <typename Enum, Enum VALUE>
+using E_t = EnumType<Enum, VALUE>;
+
+template <typename... Types>
+using FirstType_t = TypeAt_t<0, TypeList<Types...>>;
+template <typename... Types>
+using LastType_t = TypeAt_t<-1, TypeList<Types...>>;
+template <typename... IOps>
+using FirstInstantiableOperationInputType_t = typename FirstType_t<IOps...>::Operation::InputType;
+template <typename... IOps>
+using LastInstantiableOperationOutputType_t = typename LastType_t<IOps...>::Operation::OutputType;
+
+// ---- integer sequences and parameter packs -------------------------------------------------------------------------
+// Position of a value in an integer sequence (-1 when absent), and membership.
+template <typename T, T ELEMENT>
+struct Find {
+    template <T... Sequence>
+    FK_HD_STATIC int in(std::integer_sequence<T, Sequence...>) {
+        int position = -1, i = 0;
+        ((position = (position < 0 && Sequence == ELEMENT) ? i : position, ++i), ...);
+        return position;
+    }
+    template <T... Sequence>
+    FK_HD_STATIC bool one_of(std::integer_sequence<T, Sequence...>) {
+        return ((Sequence == ELEMENT) || ...);
+    }
+};
+template <typename T, T START, T... Ints>
+FK_HD_CNST auto make_integer_sequence_from(const std::integer_sequence<T, Ints...>&) {
+    return std::integer_sequence<T, (START + Ints)...>{};
+}
+template <size_t N>
+constexpr auto indexSequence = std::make_index_sequence<N>{};
+// argument INDEX of a call
+template <int INDEX, typename T, typename... Args>
+FK_HD_CNST const auto& get(const T& current, const Args&... args) {
+    static_assert(INDEX >= 0 && static_cast<int>(sizeof...(Args)) + 1 > INDEX, "Index out of range when looking for a parameter in a parameter pack.");
+    if constexpr (INDEX == 0) {
+        return current;
+    } else {
+        return get<INDEX - 1>(args...);
+    }
+}
+template <typename... Args>
+FK_HD_CNST const auto& ppFirst(const Args&... args) {
+    return get<0>(args...);
+}
+template <typename... Args>
+FK_HD_CNST const auto& ppLast(const Args&... args) {
+    return get<static_cast<int>(sizeof...(Args)) - 1>(args...);
+}
 
 // ---- filtered sequences ------------------------------------------------------------------------------------------
 // The positions of the types of a list that comply with a restriction (`Restriction::template complies<T>()`), in order.
@@ -218,7 +294,7 @@ struct TupleTypes<Tuple<Types...>> {
 template <typename TupleType>
 using ToTypeList = typename detail::TupleTypes<TupleType>::type;
 template <int INDEX, typename TupleType>
-using get_t = TypeAt_t<static_cast<size_t>(INDEX), ToTypeList<TupleType>>;
+using get_t = TypeAt_t<INDEX, ToTypeList<TupleType>>;
 
 // f(get<0>(t), get<1>(t), ...)
 namespace detail {

@@ -49,6 +49,17 @@ template <typename... Types>
 struct TypeList {
     enum { size = sizeof...(Types) };
 };
+// A TypeList of four or of six TypeLists also names their concatenation as ::type (core/utils/type_lists.h:49-59).
+template <typename... A, typename... B, typename... C, typename... D>
+struct TypeList<TypeList<A...>, TypeList<B...>, TypeList<C...>, TypeList<D...>> {
+    enum { size = 4 };
+    using type = TypeList<A..., B..., C..., D...>;
+};
+template <typename... A, typename... B, typename... C, typename... D, typename... E, typename... F>
+struct TypeList<TypeList<A...>, TypeList<B...>, TypeList<C...>, TypeList<D...>, TypeList<E...>, TypeList<F...>> {
+    enum { size = 6 };
+    using type = TypeList<A..., B..., C..., D..., E..., F...>;
+};
 
 // Throws std::runtime_error("GPU Error: <text> File: <file> Line: <line>") on a non-zero runtime status, the
 // text convention of the reference's gpuAssert (core/utils/utils.h:95-109).

@@ -95,6 +95,13 @@ FK_VECTOR_TRAITS(double, double)
 #undef FK_VECTOR_TRAITS
 
 // plain `char` maps onto the family of its signedness
+template <>
+struct VectorTraits<char> {
+    using base = std::conditional_t<std::is_unsigned_v<char>, unsigned char, signed char>;
+    static constexpr int channels = 1;
+    static constexpr bool is_vector = false;
+    enum { bytes = 1 };
+};
 template <int N>
 struct VectorType<char, N> : VectorType<std::conditional_t<std::is_unsigned_v<char>, unsigned char, signed char>, N> {};
 
@@ -111,6 +118,45 @@ constexpr int cn = VectorTraits<T>::channels;
 
 template <typename T>
 using VBase = typename VectorTraits<std::remove_cv_t<T>>::base;
+
+// ---- lists of the types above, and what may be combined with what (core/utils/cuda_vector_utils.h:74-97,308-367) -----
+template <uint CHANNELS>
+using VectorTypeList = TypeList<VectorType_t<bool, CHANNELS>, VectorType_t<uchar, CHANNELS>, VectorType_t<schar, CHANNELS>,
+                                VectorType_t<ushort, CHANNELS>, VectorType_t<short, CHANNELS>, VectorType_t<uint, CHANNELS>,
+                                VectorType_t<int, CHANNELS>, VectorType_t<ulong, CHANNELS>, VectorType_t<long, CHANNELS>,
+                                VectorType_t<ulonglong, CHANNELS>, VectorType_t<longlong, CHANNELS>, VectorType_t<float, CHANNELS>,
+                                VectorType_t<double, CHANNELS>>;
+using FloatingTypes = TypeList<float, double>;
+using IntegralTypes = TypeList<uchar, char, schar, ushort, short, uint, int, ulong, long, ulonglong, longlong>;
+using IntegralBaseTypes = TypeList<uchar, schar, ushort, short, uint, int, ulong, long, ulonglong, longlong>;
+using StandardTypes = TypeList<bool, uchar, char, schar, ushort, short, uint, int, ulong, long, ulonglong, longlong, float, double>;
+using BaseTypes = TypeList<bool, uchar, schar, ushort, short, uint, int, ulong, long, ulonglong, longlong, float, double>;
+using VOne = TypeList<bool1, uchar1, char1, ushort1, short1, uint1, int1, ulong1, long1, ulonglong1, longlong1, float1, double1>;
+using VTwo = VectorTypeList<2>;
+using VThree = VectorTypeList<3>;
+using VFour = VectorTypeList<4>;
+using VAll = typename TypeList<VOne, VTwo, VThree, VFour>::type;
+
+template <typename T>
+struct IsCudaVector : std::bool_constant<validCUDAVec<T>> {};
+template <typename I1, typename I2>
+struct BothIntegrals : std::bool_constant<std::is_integral_v<VBase<I1>> && std::is_integral_v<VBase<I2>>> {};
+template <typename I1, typename I2>
+struct AreVVEqCN : std::bool_constant<validCUDAVec<I1> && validCUDAVec<I2> && cn<I1> == cn<I2>> {};
+template <typename I1, typename I2>
+struct AreSV : std::bool_constant<std::is_fundamental_v<I1> && validCUDAVec<I2>> {};
+template <typename I1, typename I2>
+struct AreVS : std::bool_constant<validCUDAVec<I1> && std::is_fundamental_v<I2>> {};
+template <typename T>
+struct CanUnary : std::bool_constant<validCUDAVec<T>> {};
+template <typename I1, typename I2>
+struct CanBinary : std::bool_constant<AreVVEqCN<I1, I2>::value || AreSV<I1, I2>::value || AreVS<I1, I2>::value> {};
+template <typename I1, typename I2>
+struct CanBinaryBitwise : std::bool_constant<CanBinary<I1, I2>::value && BothIntegrals<I1, I2>::value> {};
+template <typename I1, typename I2>
+struct CanCompound : std::bool_constant<AreVVEqCN<I1, I2>::value || AreVS<I1, I2>::value> {};
+template <typename I1, typename I2>
+struct CanCompoundLogical : std::bool_constant<CanCompound<I1, I2>::value && BothIntegrals<I1, I2>::value> {};
 
 // ---- channel access and construction ------------------------------------------------------------------------------
 template <int I, typename T>
@@ -139,6 +185,17 @@ FK_HD_CNST VBase<T> vectorAt(int idx, const T& v) {
         if constexpr (cn<T> >= 4) { if (idx == 3) return v.w; }
         return v.x;
     }
+}
+
+// The reference's spellings of the two accessors above (core/utils/cuda_vector_utils.h:160-229).
+template <int IDX, typename T>
+FK_HD_CNST auto VectorAt(const T& v) {
+    static_assert(IDX >= 0 && IDX < cn<T>, "Index out of range for this vector type");
+    return vget<IDX>(v);
+}
+template <typename T>
+FK_HD_CNST VBase<T> VectorAt(const int& idx, const T& v) {
+    return vectorAt(idx, v);
 }
 
 // make_<T>(a, b, ...): every argument is cast to T's base type (core/utils/cuda_vector_utils.h:235-265)
@@ -212,10 +269,9 @@ FK_BINARY_FUNCTOR(FnBitXor, ^)
 #undef FK_BINARY_FUNCTOR
 
 template <typename A, typename B>
-constexpr bool can_binary = (validCUDAVec<A> && validCUDAVec<B>) || (validCUDAVec<A> && std::is_arithmetic_v<B>) ||
-                            (std::is_arithmetic_v<A> && validCUDAVec<B>);
+constexpr bool can_binary = CanBinary<A, B>::value;
 template <typename A, typename B>
-constexpr bool can_bitwise = can_binary<A, B> && std::is_integral_v<VBase<A>> && std::is_integral_v<VBase<B>>;
+constexpr bool can_bitwise = CanBinaryBitwise<A, B>::value;
 } // namespace detail
 
 } // namespace fk
@@ -244,6 +300,45 @@ FK_VEC_OPERATOR(||, FnOr, can_binary)
 FK_VEC_OPERATOR(&, FnBitAnd, can_bitwise)
 FK_VEC_OPERATOR(|, FnBitOr, can_bitwise)
 FK_VEC_OPERATOR(^, FnBitXor, can_bitwise)
+
+// Unary operators per channel; the result has the base type the scalar expression yields (a one-channel vector gives
+// that scalar itself, as in the reference), and an operator the base type does not have is not offered for its vectors.
+#define FK_VEC_UNARY(OP)                                                                                               \
+    template <typename T, std::enable_if_t<CanUnary<T>::value, int> = 0>                                               \
+    FK_HD_CNST auto operator OP(const T& a) -> VectorType_t<decltype(OP std::declval<VBase<T>>()), cn<T>> {            \
+        using O = VectorType_t<decltype(OP std::declval<VBase<T>>()), cn<T>>;                                          \
+        if constexpr (cn<T> == 1) {                                                                                    \
+            return make_<O>(OP a.x);                                                                                   \
+        } else if constexpr (cn<T> == 2) {                                                                             \
+            return make_<O>(OP a.x, OP a.y);                                                                           \
+        } else if constexpr (cn<T> == 3) {                                                                             \
+            return make_<O>(OP a.x, OP a.y, OP a.z);                                                                   \
+        } else {                                                                                                       \
+            return make_<O>(OP a.x, OP a.y, OP a.z, OP a.w);                                                           \
+        }                                                                                                              \
+    }
+FK_VEC_UNARY(-)
+FK_VEC_UNARY(!)
+FK_VEC_UNARY(~)
+#undef FK_VEC_UNARY
+
+// Compound assignment per channel: vector op= vector of the same channel count, or vector op= scalar.
+#define FK_VEC_COMPOUND(OP, COND)                                                                                      \
+    template <typename I1, typename I2, std::enable_if_t<COND<I1, I2>::value, int> = 0>                                \
+    FK_HD_CNST I1 operator OP(I1& a, const I2& b) {                                                                    \
+        a.x OP vget<0>(b);                                                                                             \
+        if constexpr (cn<I1> >= 2) a.y OP vget<1>(b);                                                                  \
+        if constexpr (cn<I1> >= 3) a.z OP vget<2>(b);                                                                  \
+        if constexpr (cn<I1> == 4) a.w OP vget<3>(b);                                                                  \
+        return a;                                                                                                      \
+    }
+FK_VEC_COMPOUND(+=, CanCompound)
+FK_VEC_COMPOUND(-=, CanCompound)
+FK_VEC_COMPOUND(*=, CanCompound)
+FK_VEC_COMPOUND(/=, CanCompound)
+FK_VEC_COMPOUND(&=, CanCompoundLogical)
+FK_VEC_COMPOUND(|=, CanCompoundLogical)
+#undef FK_VEC_COMPOUND
 } // namespace fk
 #undef FK_VEC_OPERATOR
 

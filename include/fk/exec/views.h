@@ -148,7 +148,7 @@ struct SourceOf<IOp, std::enable_if_t<ViewOf<IOp>::supported && !ViewOf<IOp>::ty
 template <typename Head, typename... ComputeOps>
 struct SourceOf<Read<FusedOperation<Head, ComputeOps...>>,
                 std::enable_if_t<isAnyReadType<Head> && ViewOf<Instantiable<Head>>::supported && !ViewOf<Instantiable<Head>>::type::IS_RESIZE &&
-                                 (sizeof...(ComputeOps) > 0)>> {
+                                 (sizeof...(ComputeOps) > 0) && noneAnyWriteType<ComputeOps...>>> {
     static constexpr bool supported = true;
     using IOp = Read<FusedOperation<Head, ComputeOps...>>;
     using View = typename ViewOf<Instantiable<Head>>::type;
@@ -225,7 +225,8 @@ struct ProgramOf<IOp, std::enable_if_t<ViewOf<IOp>::supported>> {
 };
 template <typename Head, typename... ComputeOps>
 struct ProgramOf<Read<FusedOperation<Head, ComputeOps...>>,
-                 std::enable_if_t<isAnyReadType<Head> && ViewOf<Instantiable<Head>>::supported && (sizeof...(ComputeOps) > 0)>> {
+                 std::enable_if_t<isAnyReadType<Head> && ViewOf<Instantiable<Head>>::supported && (sizeof...(ComputeOps) > 0) &&
+                                  noneAnyWriteType<ComputeOps...>>> { // a chain that writes on its way runs as a generic job
     static constexpr bool supported = true;
     using IOp = Read<FusedOperation<Head, ComputeOps...>>;
     using View = typename ViewOf<Instantiable<Head>>::type;

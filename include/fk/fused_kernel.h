@@ -3,7 +3,9 @@
 #ifndef FK_FUSED_KERNEL_H
 #define FK_FUSED_KERNEL_H
 
+#include "fk/core/array.h"
 #include "fk/core/thread_fusion_info.h"
+#include "fk/core/type_to_string.h"
 #include "fk/exec/executor.h"
 #include "fk/ops/yuv.h"
 #include "fk/ops/border_reader.h"

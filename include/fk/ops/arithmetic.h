@@ -88,9 +88,9 @@ public:
 
 
 template <typename T>
-constexpr T maxValue = std::numeric_limits<T>::max();
+constexpr T maxValue = make_set<T>(std::numeric_limits<VBase<T>>::max()); // every channel, for a vector type
 template <typename T>
-constexpr T minValue = std::numeric_limits<T>::lowest();
+constexpr T minValue = make_set<T>(std::numeric_limits<VBase<T>>::lowest());
 
 template <typename I, typename O>
 struct SaturateCastBase {

@@ -210,6 +210,52 @@ int main() {
         }
         EXPECT(ok && newest_first.nextUpdateIdx() == 7 % B);
     }
+    // 9. BatchRead -> BatchWrite: plane z of one launch is read from image z and written to its own output image
+    {
+        constexpr size_t BATCH = 3;
+        std::array<Ptr2D<uchar3>, BATCH> inputs{ Ptr2D<uchar3>(70, 9), Ptr2D<uchar3>(70, 9), Ptr2D<uchar3>(70, 9) };
+        std::array<Ptr2D<float3>, BATCH> outputs{ Ptr2D<float3>(70, 9), Ptr2D<float3>(70, 9), Ptr2D<float3>(70, 9) };
+        std::array<RawPtr<ND::_2D, float3>, BATCH> raw{};
+        for (size_t i = 0; i < BATCH; ++i) {
+            fill_ramp(inputs[i], stream, static_cast<int>(i) + 1);
+            raw[i] = outputs[i].ptr();
+        }
+        const auto writeAll = PerThreadWrite<ND::_2D, float3>::build(raw);
+        static_assert(isWriteType<std::decay_t<decltype(writeAll)>> && isBatchOperation<typename std::decay_t<decltype(writeAll)>::Operation>, "BatchWrite");
+        executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, uchar3>::build(inputs), Cast<uchar3, float3>::build(),
+                                          Mul<float3>::build(make_set<float3>(0.5f)), writeAll);
+        bool ok = true;
+        for (size_t i = 0; i < BATCH; ++i) {
+            outputs[i].download(stream);
+            stream.sync();
+            for (uint y = 0; y < 9; ++y)
+                for (uint x = 0; x < 70; ++x) ok = ok && outputs[i].at(x, y).y == 0.5f * inputs[i].at(x, y).y;
+        }
+        EXPECT(ok);
+    }
+    // 10. a write in the middle of a chain stores the value at that point and hands it on; a chain that starts with a
+    //     write is one MidWrite operation
+    {
+        Ptr2D<uchar> in(130, 7);
+        Ptr2D<float> mid(130, 7), mid2(130, 7), last(130, 7);
+        fill_ramp(in, stream, 1);
+        const auto tee = fuse(PerThreadWrite<ND::_2D, float>::build(mid2), Add<float>::build(1.f)); // write, then add
+        static_assert(isMidWriteType<std::decay_t<decltype(tee)>>, "a write-first chain is a MidWrite operation");
+        executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_2D, uchar>::build(in), Cast<uchar, float>::build(),
+                                          MidWrite<PerThreadWrite<ND::_2D, float>>{ { mid.ptr() } }, Mul<float>::build(3.f), tee,
+                                          PerThreadWrite<ND::_2D, float>::build(last));
+        mid.download(stream);
+        mid2.download(stream);
+        last.download(stream);
+        stream.sync();
+        bool ok = true;
+        for (uint y = 0; y < 7; ++y)
+            for (uint x = 0; x < 130; ++x) {
+                const float v = static_cast<float>(in.at(x, y));
+                ok = ok && mid.at(x, y) == v && mid2.at(x, y) == 3.f * v && last.at(x, y) == 3.f * v + 1.f;
+            }
+        EXPECT(ok);
+    }
     // 8. a launch the runtime rejects surfaces as the reference's exception text
     {
         bool threw = false;
