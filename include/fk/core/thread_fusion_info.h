@@ -80,6 +80,23 @@ private:
     FK_HD_STATIC BiggerWriteType join(const WriteType& a, const WriteType& b) { return make_<BiggerWriteType>(a.x, a.y, b.x, b.y); }
 };
 
+// What an operation that handles ELEMS_PER_THREAD elements of SourceType at once takes or returns: the vector of that many
+// elements when the operation passes its data through unchanged, otherwise its declared OutputType.
+namespace detail {
+template <typename SourceType, uint ELEMS_PER_THREAD, typename OutputType, typename = void>
+struct FusedElements {
+    using Wide = VectorType<VBase<SourceType>, cn<SourceType> * static_cast<int>(ELEMS_PER_THREAD)>;
+    using type = std::conditional_t<validCUDAVec<SourceType>, typename Wide::type_v, typename Wide::type>;
+};
+template <typename SourceType, uint ELEMS_PER_THREAD, typename OutputType>
+struct FusedElements<SourceType, ELEMS_PER_THREAD, OutputType,
+                     std::enable_if_t<!std::is_same_v<SourceType, OutputType> || std::is_same_v<SourceType, NullType>>> {
+    using type = OutputType;
+};
+} // namespace detail
+template <typename SourceType, uint ELEMS_PER_THREAD, typename OutputType = SourceType>
+using ThreadFusionType = typename detail::FusedElements<SourceType, ELEMS_PER_THREAD, OutputType>::type;
+
 template <bool THREAD_FUSION_ENABLED, typename... IOpTypes>
 FK_HD_CNST bool isThreadFusionEnabled() {
     using ReadOperation = typename TypeAt_t<0, TypeList<IOpTypes...>>::Operation;

@@ -4,6 +4,7 @@
 #define FK_FUSED_KERNEL_H
 
 #include "fk/core/array.h"
+#include "fk/core/parent_operations.h"
 #include "fk/core/thread_fusion_info.h"
 #include "fk/core/type_to_string.h"
 #include "fk/exec/executor.h"

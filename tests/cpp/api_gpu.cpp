@@ -26,6 +26,65 @@ static void fill_ramp(Ptr2D<T>& img, Stream& stream, int scale) {
     img.upload(stream);
 }
 
+// Operations written by a user in the style of the Fused Kernel Library: a Parent names the member types, the DECLARE
+// macro imports them (parent_operations.h of the reference).  One of each kind that a chain can hold.
+template <typename T>
+struct UserMirrorRead { // reads the row back to front
+private:
+    using SelfType = UserMirrorRead<T>;
+
+public:
+    FK_STATIC_STRUCT(UserMirrorRead, SelfType)
+    using Parent = ReadOperation<T, RawPtr<ND::_2D, T>, T, TF::DISABLED, UserMirrorRead<T>>;
+    DECLARE_READ_PARENT
+    FK_HOST_DEVICE_FUSE OutputType exec(const Point& thread, const ParamsType& params) {
+        return *PtrAccessor<ND::_2D>::cr_point(Point(static_cast<int>(params.dims.width) - 1 - thread.x, thread.y), params);
+    }
+    FK_HOST_DEVICE_FUSE uint num_elems_x(const Point&, const OperationDataType& opData) { return opData.params.dims.width; }
+    FK_HOST_DEVICE_FUSE uint num_elems_y(const Point&, const OperationDataType& opData) { return opData.params.dims.height; }
+    FK_HOST_DEVICE_FUSE uint num_elems_z(const Point&, const OperationDataType&) { return 1; }
+    FK_HOST_DEVICE_FUSE ActiveThreads getActiveThreads(const OperationDataType& opData) {
+        return ActiveThreads(opData.params.dims.width, opData.params.dims.height, 1);
+    }
+};
+template <typename T>
+struct UserSquare {
+private:
+    using SelfType = UserSquare<T>;
+
+public:
+    FK_STATIC_STRUCT(UserSquare, SelfType)
+    using Parent = UnaryOperation<T, T, UserSquare<T>>;
+    DECLARE_UNARY_PARENT
+    FK_HOST_DEVICE_FUSE OutputType exec(const InputType& input) { return input * input; }
+};
+template <typename T>
+struct UserAxpy { // a * x + b with { a, b } as parameters
+private:
+    using SelfType = UserAxpy<T>;
+
+public:
+    FK_STATIC_STRUCT(UserAxpy, SelfType)
+    using Parent = BinaryOperation<T, Tuple<T, T>, T, UserAxpy<T>>;
+    DECLARE_BINARY_PARENT
+    FK_HOST_DEVICE_FUSE OutputType exec(const InputType& input, const ParamsType& params) { return get<0>(params) * input + get<1>(params); }
+};
+template <typename T>
+struct UserTransposedWrite {
+private:
+    using SelfType = UserTransposedWrite<T>;
+
+public:
+    FK_STATIC_STRUCT(UserTransposedWrite, SelfType)
+    using Parent = WriteOperation<T, RawPtr<ND::_2D, T>, T, TF::DISABLED, UserTransposedWrite<T>>;
+    DECLARE_WRITE_PARENT
+    FK_HOST_DEVICE_FUSE void exec(const Point& thread, const InputType& input, const ParamsType& params) {
+        *PtrAccessor<ND::_2D>::point(Point(thread.y, thread.x), params) = input;
+    }
+    FK_HOST_DEVICE_FUSE uint num_elems_x(const Point&, const OperationDataType& opData) { return opData.params.dims.width; }
+    FK_HOST_DEVICE_FUSE uint pitch(const Point&, const OperationDataType& opData) { return opData.params.dims.pitch; }
+};
+
 int main() {
     Stream stream;
     Stream alias = stream; // copies share the native stream
@@ -253,6 +312,25 @@ int main() {
             for (uint x = 0; x < 130; ++x) {
                 const float v = static_cast<float>(in.at(x, y));
                 ok = ok && mid.at(x, y) == v && mid2.at(x, y) == 3.f * v && last.at(x, y) == 3.f * v + 1.f;
+            }
+        EXPECT(ok);
+    }
+    // 11. user-defined operations of every kind in one chain, between library operations
+    {
+        constexpr uint W = 77, H = 13;
+        Ptr2D<float> in(W, H), out(H, W);
+        for (uint y = 0; y < H; ++y)
+            for (uint x = 0; x < W; ++x) in.at(x, y) = static_cast<float>(x) - 0.25f * static_cast<float>(y);
+        in.upload(stream);
+        executeOperations<TransformDPP<>>(stream, UserMirrorRead<float>::build(in.ptr()), UserSquare<float>::build(), Add<float>::build(1.f),
+                                          UserAxpy<float>::build(Tuple<float, float>{ 2.f, -3.f }), UserTransposedWrite<float>::build(out.ptr()));
+        out.download(stream);
+        stream.sync();
+        bool ok = true;
+        for (uint y = 0; y < H; ++y)
+            for (uint x = 0; x < W; ++x) {
+                const float v = in.at(W - 1 - x, y);
+                ok = ok && out.at(y, x) == 2.f * (v * v + 1.f) + -3.f;
             }
         EXPECT(ok);
     }
