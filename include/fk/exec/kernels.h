@@ -223,7 +223,10 @@ struct SourceAccess<PlainView<T>> {
     __device__ __attribute__((always_inline)) static inline const char* row(const View& v, int y) {
         return reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy + y) * v.pitch + static_cast<size_t>(v.ox) * sizeof(T);
     }
-    __device__ __attribute__((always_inline)) static inline T load_one(const View& v, int x, int y) { return reinterpret_cast<const T*>(row(v, y))[x]; }
+    __device__ __attribute__((always_inline)) static inline T load_one(const View& v, int x, int y) {
+        // element v.ox + x of a buffer row that holds at least v.ox + v.w elements
+        return fk::detail::read_element(reinterpret_cast<const T*>(row(v, y)) + x, v.ox + x, static_cast<uint>(v.ox + v.w));
+    }
     template <int K>
     __device__ __attribute__((always_inline)) static inline void load_group(const View& v, int x0, int y, T* out) {
         constexpr int NB = K * static_cast<int>(sizeof(T));
@@ -717,6 +720,9 @@ struct ResizeJob {
 };
 
 // ---- generic -----------------------------------------------------------------------------------------------------
+// One element per thread, a block covers 64 x 4 of them.  (Several elements per thread do not pay here: the reads of an
+// arbitrary chain sit behind its own branches - border arithmetic, bounds checks - so they do not overlap, and the
+// smaller grid costs medium-sized outputs their last round of waves.)
 template <typename Sender, typename Receiver>
 struct GenericJob {
     static constexpr bool READ_IN_PLACE = isBatchOperation<typename Sender::Operation> || isBatchOperation<typename Receiver::Operation>;
@@ -725,6 +731,7 @@ struct GenericJob {
     ActiveThreads active;
     unsigned grid_x, grid_y;
     size_t lds_bytes() const { return 0; }
+    static unsigned blocks_x(unsigned width) { return (width + 63u) / 64u; }
 
     __device__ __attribute__((always_inline)) static inline void run(const GenericJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char*) {
         const int tid = dev::thread_in_block();

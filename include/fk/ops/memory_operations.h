@@ -37,7 +37,9 @@ public:
     static constexpr bool THREAD_FUSION = true;
     static constexpr ND DIMS = D;
 
-    FK_HD_STATIC OutputType exec(const Point& thread, const ParamsType& params) { return *PtrAccessor<D>::cr_point(thread, params); }
+    FK_HD_STATIC OutputType exec(const Point& thread, const ParamsType& params) {
+        return fk::detail::read_element(PtrAccessor<D>::cr_point(thread, params), thread.x, params.dims.width);
+    }
     FK_HD_STATIC OutputType exec(const Point& thread, const OperationDataType& opData) { return exec(thread, opData.params); }
     FK_HD_STATIC uint num_elems_x(const Point&, const OperationDataType& opData) { return opData.params.dims.width; }
     FK_HD_STATIC uint num_elems_y(const Point&, const OperationDataType& opData) {
@@ -112,7 +114,9 @@ public:
     static constexpr bool IS_FUSED_OP = false;
     static constexpr bool THREAD_FUSION = true;
 
-    FK_HD_STATIC OutputType exec(const Point& thread, const ParamsType& params) { return *PtrAccessor<ND::_3D>::cr_point(thread, params); }
+    FK_HD_STATIC OutputType exec(const Point& thread, const ParamsType& params) {
+        return fk::detail::read_element(PtrAccessor<ND::_3D>::cr_point(thread, params), thread.x, params.dims.width);
+    }
     FK_HD_STATIC OutputType exec(const Point& thread, const OperationDataType& opData) { return exec(thread, opData.params); }
     FK_HD_STATIC uint num_elems_x(const Point&, const OperationDataType& opData) { return opData.params.dims.width; }
     FK_HD_STATIC uint num_elems_y(const Point&, const OperationDataType& opData) { return opData.params.dims.height; }
