@@ -668,7 +668,12 @@ struct ResizeJob {
             interior = interior && tx0 + v.off_x >= v.x1 && tx0 + RESIZE_TILE_W - 1 + v.off_x <= v.x2 && ty0 + v.off_y >= v.y1 &&
                        ty0 + RESIZE_TILE_H - 1 + v.off_y <= v.y2;
         }
-        if (staged) {
+        if (!resamples) {
+            // a tile that lies wholly beside the image (the bars of a preserved aspect ratio): one value for all of it
+            const OutPixel bar = dev::apply_tail(prog.tail, v.background);
+#pragma unroll
+            for (int k = 0; k < RESIZE_PX; ++k) o[k] = bar;
+        } else if (staged) {
             if (interior) pixels<true, true>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
             else pixels<true, false>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
         } else {

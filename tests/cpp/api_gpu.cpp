@@ -6,6 +6,7 @@
 
 #include <cmath>
 #include <cstdio>
+#include <cstring>
 
 using namespace fk;
 
@@ -333,6 +334,44 @@ int main() {
                 ok = ok && out.at(y, x) == 2.f * (v * v + 1.f) + -3.f;
             }
         EXPECT(ok);
+    }
+    // 12. Div on the GPU gives the results of the IEEE division for every float (the kernels are built without fast-math
+    //     and keep subnormals): random bit patterns, subnormal operands and results, exact ties among subnormal results
+    //     (x = k * 2^-149 * d), infinities, NaNs and signed zeros
+    {
+        const uint N = 1u << 20;
+        Ptr1D<float> in(N), out(N);
+        unsigned long long state = 42;
+        const auto next = [&state]() {
+            state += 0x9E3779B97F4A7C15ull;
+            unsigned long long z = state;
+            z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+            z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+            return static_cast<unsigned>(z ^ (z >> 31));
+        };
+        int mismatches = 0;
+        for (const float d : { 255.f, 6.f, 0.229f, 1e-30f, 3e38f, -7.f, 5e-39f, 1.f / 3.f }) {
+            for (uint i = 0; i < N; ++i) {
+                unsigned bits = next();
+                if (i % 4 == 1) bits &= 0x807fffffu;                        // subnormal operands
+                if (i % 4 == 2) bits = (bits & 0x80ffffffu) | 0x00800000u; // smallest normal operands
+                if (i % 64 == 3) bits = (i / 64 % 4 == 0) ? 0x7f800000u : (i / 64 % 4 == 1) ? 0xff800000u : (i / 64 % 4 == 2) ? 0x7fc00000u : 0x80000000u;
+                float v;
+                std::memcpy(&v, &bits, 4);
+                if (i % 4 == 3 && i < 4096) v = static_cast<float>(i / 4) * 1.40129846e-45f * d;
+                in.at(i) = v;
+            }
+            in.upload(stream);
+            executeOperations<TransformDPP<>>(stream, PerThreadRead<ND::_1D, float>::build(in), Div<float>::build(d), PerThreadWrite<ND::_1D, float>::build(out));
+            out.download(stream);
+            stream.sync();
+            for (uint i = 0; i < N; ++i) {
+                const volatile float x = in.at(i), divisor = d; // volatile: the host compiler must divide, not fold
+                const float want = x / divisor, got = out.at(i);
+                if (std::memcmp(&want, &got, 4) != 0 && !(std::isnan(want) && std::isnan(got))) ++mismatches;
+            }
+        }
+        EXPECT(mismatches == 0);
     }
     // 8. a launch the runtime rejects surfaces as the reference's exception text
     {
