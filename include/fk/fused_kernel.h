@@ -17,36 +17,12 @@
 
 namespace fk {
 
+// executeOperations<DPP>(...) with any of the argument lists Executor<DPP>::executeOperations accepts: a stream and a
+// chain of IOps; an input buffer (or an array of them, optionally with the number of used planes and a default value), an
+// optional output buffer or tensor, the stream and the compute operations between them.
 template <typename DPPType, typename... Args>
-inline void executeOperations(Stream_<DPPType::PAR_ARCH>& stream, const Args&... args) {
-    Executor<DPPType>::executeOperations(stream, args...);
-}
-template <typename DPPType, ND D, typename I, typename... Args>
-inline void executeOperations(const Ptr<D, I>& input, Stream_<DPPType::PAR_ARCH>& stream, const Args&... args) {
-    Executor<DPPType>::executeOperations(input, stream, args...);
-}
-template <typename DPPType, ND D, typename I, typename O, typename... Args>
-inline void executeOperations(const Ptr<D, I>& input, const Ptr<D, O>& output, Stream_<DPPType::PAR_ARCH>& stream, const Args&... args) {
-    Executor<DPPType>::executeOperations(input, output, stream, args...);
-}
-template <typename DPPType, typename I, size_t BATCH, typename... Args>
-inline void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, const int& activeBatch, const I& defaultValue,
-                              Stream_<DPPType::PAR_ARCH>& stream, const Args&... args) {
-    Executor<DPPType>::executeOperations(input, activeBatch, defaultValue, stream, args...);
-}
-template <typename DPPType, typename I, size_t BATCH, typename... Args>
-inline void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, Stream_<DPPType::PAR_ARCH>& stream, const Args&... args) {
-    Executor<DPPType>::executeOperations(input, stream, args...);
-}
-template <typename DPPType, typename I, typename O, size_t BATCH, typename... Args>
-inline void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, const int& activeBatch, const I& defaultValue,
-                              const Tensor<O>& output, Stream_<DPPType::PAR_ARCH>& stream, const Args&... args) {
-    Executor<DPPType>::executeOperations(input, activeBatch, defaultValue, output, stream, args...);
-}
-template <typename DPPType, typename I, typename O, size_t BATCH, typename... Args>
-inline void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, const Tensor<O>& output,
-                              Stream_<DPPType::PAR_ARCH>& stream, const Args&... args) {
-    Executor<DPPType>::executeOperations(input, output, stream, args...);
+inline void executeOperations(Args&&... args) {
+    Executor<DPPType>::executeOperations(std::forward<Args>(args)...);
 }
 
 // Fills a buffer with one value: on the device through the fused executor, and its host mirror directly.

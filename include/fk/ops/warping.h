@@ -25,8 +25,15 @@ struct WarpingParameters<WarpType::Perspective> {
     Size dstSize;
 };
 
-// Source coordinate of a destination pixel: (m00*x + m01*y) + m02 and so on, each product and sum in float, and for
-// the perspective case the result multiplied by 1 / ((m20*x + m21*y) + m22).
+namespace detail {
+// (r0 * x + r1 * y) + r2, every product and sum rounded to float: one row of the matrix applied to a pixel position
+FK_HD_CNST float warp_row(const float (&row)[3], const int x, const int y) {
+    return row[0] * x + row[1] * y + row[2];
+}
+} // namespace detail
+
+// Source coordinate of a destination pixel; for the perspective case the first two rows are multiplied by the reciprocal
+// of the third (a float division, then two multiplications).
 template <WarpType WT>
 struct WarpingCoords {
 private:
@@ -35,17 +42,13 @@ private:
 public:
     FK_BINARY_OPERATION(WarpingCoords, Point, WarpingParameters<WT>, float2)
     FK_HD_STATIC OutputType exec(const InputType& thread, const ParamsType& params) {
-        const int x = thread.x;
-        const int y = thread.y;
-        const auto& m = params.transformMatrix.data;
-        const float xs = m[0][0] * x + m[0][1] * y + m[0][2];
-        const float ys = m[1][0] * x + m[1][1] * y + m[1][2];
+        const auto& matrix = params.transformMatrix.data;
+        float2 source{ detail::warp_row(matrix[0], thread.x, thread.y), detail::warp_row(matrix[1], thread.x, thread.y) };
         if constexpr (WT == WarpType::Perspective) {
-            const float coeff = 1.0f / (m[2][0] * x + m[2][1] * y + m[2][2]);
-            return float2{ coeff * xs, coeff * ys };
-        } else {
-            return float2{ xs, ys };
+            const float scale = 1.0f / detail::warp_row(matrix[2], thread.x, thread.y);
+            source = float2{ scale * source.x, scale * source.y };
         }
+        return source;
     }
 };
 
