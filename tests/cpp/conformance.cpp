@@ -4,6 +4,8 @@
 // 49-116, tests/operation/test_operation_types.h:56-182, tests/data/test_rect.h:19-39, tests/data/test_ptr_nd.h:44-108).
 // Needs no GPU: everything here is compile-time or host memory.  Exit code 0 = pass.
 #include <fused_kernel/fused_kernel.h>
+#include <fused_kernel/fused_kernel.cuh> // the spelling the reference's README still uses
+#include <fused_kernel/algorithms/image_processing/resize.cuh>
 
 #include <cstdio>
 #include <cstring>
