@@ -89,9 +89,9 @@ def build_benchmarks():
 
 
 # The reference's own test headers that exercise this path's operator API (relative to the reference checkout); each
-# defines `int launch()`.  Left out: examples/readme_test_code.h (half of it runs on the reference's CPU backend), the
-# string tests (text rendering of operations, not part of this path) and benchmarks/ (their timing harness is written
-# against the CUDA runtime's event and stream types; fusedkernellibrary_amd/benchmarks/reference_sweeps.cpp restates them).
+# defines `int launch()`.  Left out: examples/readme_test_code.h (half of it runs on the reference's CPU backend),
+# cudabug/ (nvcc bug reproducers) and benchmarks/ (their timing harness is written against the CUDA runtime's event and
+# stream types; fusedkernellibrary_amd/benchmarks/reference_sweeps.cpp restates them).
 REFERENCE_TESTS = (
     "tests/algorithm/test_batchresize_build.h", "tests/algorithm/test_border_reader.h", "tests/algorithm/test_crop.h",
     "tests/algorithm/test_deinterlace.h", "tests/algorithm/test_warp.h", "tests/data/test_ptr_nd.h", "tests/data/test_rect.h",
@@ -102,6 +102,8 @@ REFERENCE_TESTS = (
     "utests/algorithm/image_processing/utest_saturate.h", "utests/algorithm/image_processing/utest_color_conversion.h",
     "utests/algorithm/image_processing/utest_deinterlace.h", "utests/core/constexpr_libs/utest_constexpr_cmath.h",
     "utests/core/utils/utest_VBase.h", "utests/core/utils/utest_cuda_vector_utils.h",
+    "tests/string/test_fk_string.h", "tests/string/test_IOps_to_string.h", "tests/string/test_literal_to_string.h",
+    "tests/string/test_struct_to_string.h",
 )
 REFERENCE_ROOT = os.environ.get("FK_REFERENCE_ROOT", "/root/reference")
 REFERENCE_TESTS_DIR = os.path.join(ROOT, "tests", "cpp", "reference_tests")

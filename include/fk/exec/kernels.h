@@ -576,12 +576,13 @@ struct ResizeJob {
                     c = dev::slot_to_pixel<Src>(sc);
                     d = dev::slot_to_pixel<Src>(sd);
                 } else if constexpr (RAW_SOURCE) {
-                    const char* const r0 = window + static_cast<size_t>(t.y1) * s.pitch;
-                    const char* const r1 = window + static_cast<size_t>(t.y2r) * s.pitch;
-                    a = reinterpret_cast<const Src*>(r0)[t.x1];
-                    b = reinterpret_cast<const Src*>(r0)[t.x2r];
-                    c = reinterpret_cast<const Src*>(r1)[t.x1];
-                    d = reinterpret_cast<const Src*>(r1)[t.x2r];
+                    const Src* const r0 = reinterpret_cast<const Src*>(window + static_cast<size_t>(t.y1) * s.pitch);
+                    const Src* const r1 = reinterpret_cast<const Src*>(window + static_cast<size_t>(t.y2r) * s.pitch);
+                    const uint row_elems = static_cast<uint>(s.ox + s.w); // the buffer row holds at least the window
+                    a = fk::detail::read_element(r0 + t.x1, s.ox + t.x1, row_elems);
+                    b = fk::detail::read_element(r0 + t.x2r, s.ox + t.x2r, row_elems);
+                    c = fk::detail::read_element(r1 + t.x1, s.ox + t.x1, row_elems);
+                    d = fk::detail::read_element(r1 + t.x2r, s.ox + t.x2r, row_elems);
                 } else {
                     a = fetch(v, t.x1, t.y1);
                     b = fetch(v, t.x2r, t.y1);

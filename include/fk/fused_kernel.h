@@ -6,6 +6,7 @@
 #include "fk/core/array.h"
 #include "fk/core/parent_operations.h"
 #include "fk/core/thread_fusion_info.h"
+#include "fk/core/string.h"
 #include "fk/core/type_to_string.h"
 #include "fk/exec/executor.h"
 #include "fk/ops/yuv.h"
