@@ -89,8 +89,8 @@ def build_benchmarks():
 
 
 # The reference's own test headers that exercise this path's operator API (relative to the reference checkout); each
-# defines `int launch()`.  Left out: examples/readme_test_code.h (half of it runs on the reference's CPU backend),
-# cudabug/ (nvcc bug reproducers) and benchmarks/ (their timing harness is written against the CUDA runtime's event and
+# defines `int launch()`.  Left out: examples/readme_test_code.h (half of it runs on the reference's CPU backend) and
+# benchmarks/ (their timing harness is written against the CUDA runtime's event and
 # stream types; fusedkernellibrary_amd/benchmarks/reference_sweeps.cpp restates them).
 REFERENCE_TESTS = (
     "tests/algorithm/test_batchresize_build.h", "tests/algorithm/test_border_reader.h", "tests/algorithm/test_crop.h",
@@ -104,6 +104,7 @@ REFERENCE_TESTS = (
     "utests/core/utils/utest_VBase.h", "utests/core/utils/utest_cuda_vector_utils.h",
     "tests/string/test_fk_string.h", "tests/string/test_IOps_to_string.h", "tests/string/test_literal_to_string.h",
     "tests/string/test_struct_to_string.h",
+    "tests/cudabug/test_nvcc124_126_BugReproducer.h", "tests/cudabug/test_nvcc1281_129_BugReproducer.h",
 )
 REFERENCE_ROOT = os.environ.get("FK_REFERENCE_ROOT", "/root/reference")
 REFERENCE_TESTS_DIR = os.path.join(ROOT, "tests", "cpp", "reference_tests")
