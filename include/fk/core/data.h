@@ -193,21 +193,23 @@ struct PtrAccessor<ND::T3D> {
 };
 
 namespace detail {
-// Element x of a row, given its address.  On the GPU a pixel of three one-byte channels is fetched with one (unaligned)
-// dword load instead of three byte loads: a wave's memory instructions cost the same address-processing time whatever
-// their width, and kernels that gather such pixels one by one are bound by exactly that.  The dword starts one byte
-// early for every element but the first of its row, so it never reaches past the row's last element; a row of a single
-// element takes the plain path.
+// The element at `p`.  On the GPU a pixel of three one-byte channels is fetched with one (unaligned) dword load instead of
+// three byte loads: a wave's memory instructions cost the same address-processing time whatever their width, and kernels
+// that gather such pixels one by one are bound by exactly that.  The dword is [p, p + 4) when p is dword-aligned and
+// [p - 1, p + 3) otherwise; either way its one byte that is not the pixel's lies in an aligned dword that also holds a
+// byte of the pixel, so it is on the pixel's own page: the load cannot fault wherever the buffer begins or ends, and it
+// needs no branch, so the taps of an interpolation are in flight together.
 template <typename T>
-FK_HD_CNST T read_element(const T* p, const int x, const uint width) {
+FK_HD_CNST T read_element(const T* p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     if constexpr (validCUDAVec<T> && cn<T> == 3 && sizeof(T) == 3) {
-        if (!__builtin_is_constant_evaluated() && width >= 2) {
+        if (!__builtin_is_constant_evaluated()) {
             using B = VBase<T>;
-            const int back = x > 0 ? 1 : 0;
+            const unsigned char* const bytes = reinterpret_cast<const unsigned char*>(p);
+            const unsigned back = (static_cast<unsigned>(reinterpret_cast<size_t>(bytes)) & 3u) != 0u ? 1u : 0u;
             unsigned int w = 0;
-            __builtin_memcpy(&w, reinterpret_cast<const unsigned char*>(p) - back, 4);
-            w >>= 8 * back;
+            __builtin_memcpy(&w, bytes - back, 4);
+            w >>= 8u * back;
             return T{ static_cast<B>(static_cast<unsigned char>(w)), static_cast<B>(static_cast<unsigned char>(w >> 8)),
                       static_cast<B>(static_cast<unsigned char>(w >> 16)) };
         }

@@ -224,8 +224,7 @@ struct SourceAccess<PlainView<T>> {
         return reinterpret_cast<const char*>(v.data) + static_cast<size_t>(v.oy + y) * v.pitch + static_cast<size_t>(v.ox) * sizeof(T);
     }
     __device__ __attribute__((always_inline)) static inline T load_one(const View& v, int x, int y) {
-        // element v.ox + x of a buffer row that holds at least v.ox + v.w elements
-        return fk::detail::read_element(reinterpret_cast<const T*>(row(v, y)) + x, v.ox + x, static_cast<uint>(v.ox + v.w));
+        return fk::detail::read_element(reinterpret_cast<const T*>(row(v, y)) + x);
     }
     template <int K>
     __device__ __attribute__((always_inline)) static inline void load_group(const View& v, int x0, int y, T* out) {
@@ -578,11 +577,10 @@ struct ResizeJob {
                 } else if constexpr (RAW_SOURCE) {
                     const Src* const r0 = reinterpret_cast<const Src*>(window + static_cast<size_t>(t.y1) * s.pitch);
                     const Src* const r1 = reinterpret_cast<const Src*>(window + static_cast<size_t>(t.y2r) * s.pitch);
-                    const uint row_elems = static_cast<uint>(s.ox + s.w); // the buffer row holds at least the window
-                    a = fk::detail::read_element(r0 + t.x1, s.ox + t.x1, row_elems);
-                    b = fk::detail::read_element(r0 + t.x2r, s.ox + t.x2r, row_elems);
-                    c = fk::detail::read_element(r1 + t.x1, s.ox + t.x1, row_elems);
-                    d = fk::detail::read_element(r1 + t.x2r, s.ox + t.x2r, row_elems);
+                    a = fk::detail::read_element(r0 + t.x1);
+                    b = fk::detail::read_element(r0 + t.x2r);
+                    c = fk::detail::read_element(r1 + t.x1);
+                    d = fk::detail::read_element(r1 + t.x2r);
                 } else {
                     a = fetch(v, t.x1, t.y1);
                     b = fetch(v, t.x2r, t.y1);

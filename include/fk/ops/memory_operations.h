@@ -38,7 +38,7 @@ public:
     static constexpr ND DIMS = D;
 
     FK_HD_STATIC OutputType exec(const Point& thread, const ParamsType& params) {
-        return fk::detail::read_element(PtrAccessor<D>::cr_point(thread, params), thread.x, params.dims.width);
+        return fk::detail::read_element(PtrAccessor<D>::cr_point(thread, params));
     }
     FK_HD_STATIC OutputType exec(const Point& thread, const OperationDataType& opData) { return exec(thread, opData.params); }
     FK_HD_STATIC uint num_elems_x(const Point&, const OperationDataType& opData) { return opData.params.dims.width; }
@@ -115,7 +115,7 @@ public:
     static constexpr bool THREAD_FUSION = true;
 
     FK_HD_STATIC OutputType exec(const Point& thread, const ParamsType& params) {
-        return fk::detail::read_element(PtrAccessor<ND::_3D>::cr_point(thread, params), thread.x, params.dims.width);
+        return fk::detail::read_element(PtrAccessor<ND::_3D>::cr_point(thread, params));
     }
     FK_HD_STATIC OutputType exec(const Point& thread, const OperationDataType& opData) { return exec(thread, opData.params); }
     FK_HD_STATIC uint num_elems_x(const Point&, const OperationDataType& opData) { return opData.params.dims.width; }
