@@ -165,7 +165,7 @@ struct JobOf {
             job.sender = sender;
             job.receiver = receiver;
             job.active = sender.getActiveThreads();
-            job.grid_x = decltype(job)::blocks_x(job.active.x);
+            job.grid_x = job.plan(job.active);
             job.grid_y = ceil_div(job.active.y, 4u);
             return job;
         }

@@ -724,27 +724,51 @@ struct ResizeJob {
 };
 
 // ---- generic -----------------------------------------------------------------------------------------------------
-// One element per thread, a block covers 64 x 4 of them.  (Several elements per thread do not pay here: the reads of an
-// arbitrary chain sit behind its own branches - border arithmetic, bounds checks - so they do not overlap, and the
-// smaller grid costs medium-sized outputs their last round of waves.)
+// A block covers 64*K x 4 elements; a thread computes K elements of one row, 64 apart (each of a wave's memory
+// instructions still covers 64 neighbours).  A chain that only gathers and stores is bound by the memory round trip, one
+// gather in flight per wave; with K = 4 a thread issues the reads of four elements before it uses any of them, provided
+// the chain's read is straight-line code (lanes past the end of a row read its last element again instead of branching
+// around the read).  K = 1 is kept for small outputs, which need every wave they can get.
+constexpr unsigned GENERIC_WIDE_MIN_ELEMS = 1u << 22;
 template <typename Sender, typename Receiver>
 struct GenericJob {
     static constexpr bool READ_IN_PLACE = isBatchOperation<typename Sender::Operation> || isBatchOperation<typename Receiver::Operation>;
+    using Value = std::decay_t<decltype(Sender::Operation::exec(Point(), std::declval<const Sender&>()))>;
     Sender sender;
     Receiver receiver;
     ActiveThreads active;
     unsigned grid_x, grid_y;
+    unsigned wide; // 4 elements per thread instead of 1
     size_t lds_bytes() const { return 0; }
-    static unsigned blocks_x(unsigned width) { return (width + 63u) / 64u; }
+    // decides the elements per thread from the size of the output and returns the number of blocks along x
+    unsigned plan(const ActiveThreads& extent) {
+        const size_t elems = static_cast<size_t>(extent.x) * extent.y * extent.z;
+        wide = (elems >= GENERIC_WIDE_MIN_ELEMS && extent.x >= 256u) ? 1u : 0u;
+        const unsigned tile_w = wide != 0u ? 256u : 64u;
+        return (extent.x + tile_w - 1u) / tile_w;
+    }
 
-    __device__ __attribute__((always_inline)) static inline void run(const GenericJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char*) {
+    template <int K>
+    __device__ __attribute__((always_inline)) static inline void body(const GenericJob& job, unsigned bx, unsigned by, unsigned bz) {
         const int tid = dev::thread_in_block();
-        const int x = static_cast<int>(bx) * 64 + (tid & 63);
+        const int x0 = static_cast<int>(bx) * (64 * K) + (tid & 63);
         const int y = static_cast<int>(by) * 4 + (tid >> 6);
-        if (x >= static_cast<int>(job.active.x) || y >= static_cast<int>(job.active.y)) return;
-        const Point thread(x, y, static_cast<int>(bz));
-        const auto value = Sender::Operation::exec(thread, job.sender);
-        Receiver::Operation::exec(thread, value, job.receiver);
+        const int w = static_cast<int>(job.active.x);
+        if (x0 >= w || y >= static_cast<int>(job.active.y)) return;
+        Value value[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const int x = x0 + 64 * k < w ? x0 + 64 * k : w - 1;
+            value[k] = Sender::Operation::exec(Point(x, y, static_cast<int>(bz)), job.sender);
+        }
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            if (x0 + 64 * k < w) Receiver::Operation::exec(Point(x0 + 64 * k, y, static_cast<int>(bz)), value[k], job.receiver);
+        }
+    }
+    __device__ __attribute__((always_inline)) static inline void run(const GenericJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char*) {
+        if (job.wide != 0u) body<4>(job, bx, by, bz);
+        else body<1>(job, bx, by, bz);
     }
 };
 

@@ -74,10 +74,12 @@ public:
         const float2 coord = WarpingCoords<WT>::exec(thread, params);
         const Size sourceSize(static_cast<int>(BackIOp::Operation::num_elems_x(thread, backIOp)),
                               static_cast<int>(BackIOp::Operation::num_elems_y(thread, backIOp)));
-        if (coord.x >= 0.f && coord.x < sourceSize.width && coord.y >= 0.f && coord.y < sourceSize.height) {
-            return Interpolate<InterpolationType::INTER_LINEAR, BackIOp>::exec(coord, { sourceSize }, backIOp);
-        }
-        return make_set<OutputType>(0.f);
+        const bool inside = coord.x >= 0.f && coord.x < sourceSize.width && coord.y >= 0.f && coord.y < sourceSize.height;
+        // A position outside the source samples nothing and yields zero.  It is moved to the origin so that the sample
+        // can be taken without a branch: straight-line code lets the reads of neighbouring work overlap on a GPU.
+        const float2 position = inside ? coord : float2{ 0.f, 0.f };
+        const OutputType sample = Interpolate<InterpolationType::INTER_LINEAR, BackIOp>::exec(position, { sourceSize }, backIOp);
+        return inside ? sample : make_set<OutputType>(0.f);
     }
     FK_HD_STATIC OutputType exec(const Point& thread, const OperationDataType& opData) { return exec(thread, opData.params, opData.backIOp); }
     FK_HD_STATIC uint num_elems_x(const Point&, const OperationDataType& opData) { return static_cast<uint>(opData.params.dstSize.width); }
