@@ -117,6 +117,28 @@ def test_full_frame_properties(fk, oracle):
     assert torch.equal(c[32:-32, 32:-32], d_src) and torch.equal(c[:32, 32:-32], torch.flip(d_src[1:33], dims=(0,)))
 
 
+def test_large_outputs_vs_oracle(fk, oracle):
+    """Outputs of 4 M elements and more run four elements per thread: a rotation and a perspective map into 2601 x 1701
+    (a width that is no multiple of the 256-element tile, rows padded) and a reflected border, element for element."""
+    import math
+    w, h = 1930, 1090
+    src = oracle.bytes(123, (h, w, 3))
+    d_src = dev(src, 5)
+    dst = (2601, 1701)
+    a = math.radians(7.0)
+    maps = [(B.WARP_AFFINE, [[math.cos(a) * 0.7, -math.sin(a) * 0.7, 40.0], [math.sin(a) * 0.7, math.cos(a) * 0.7, -150.0]]),
+            (B.WARP_PERSPECTIVE, [[0.8, 0.02, -30.0], [0.01, 0.7, 10.0], [1e-5, -2e-5, 1.0]])]
+    for wt, m in maps:
+        out = out_f32(*dst, 3)
+        fk.warp_u8c3_f32c3(wt, m, d_src, out)
+        torch.cuda.synchronize()
+        assert same_bits(host(out), oracle.warp_u8c3_f32c3(wt, m, src, dst)), wt
+    big = out_u8(w + 2 * 300, h + 2 * 300, 7)
+    fk.border_crop_u8c3(B.BORDER_REFLECT, d_src, 300, 300, big)
+    torch.cuda.synchronize()
+    assert same_bits(host(big), oracle.border_crop_u8c3(B.BORDER_REFLECT, src, 300, 300, (w + 600, h + 600)))
+
+
 def test_argument_errors(fk):
     src = torch.zeros((8, 8, 3), dtype=torch.uint8, device="cuda")
     with pytest.raises(fk.FkError, match="unsupported"):
