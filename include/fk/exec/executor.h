@@ -158,6 +158,14 @@ struct JobOf {
                 job.tx_shift = shift;
                 job.grid_x = ceil_div(groups, 1u << shift);
                 job.grid_y = ceil_div(static_cast<unsigned>(max_h), BLOCK_THREADS >> shift);
+                job.pair_limit = 0u;
+                if constexpr (N == 1 && Access::PAIRS_ROWS) {
+                    // one row per block row: rows that share a chroma row are handed to the same XCD
+                    if (shift == 8u) {
+                        const unsigned total = job.grid_x * job.grid_y, unit = 16u * job.grid_x; // whole turns of all XCDs, whole row pairs
+                        job.pair_limit = total / unit * unit;
+                    }
+                }
                 return job;
             }
         } else {

@@ -216,6 +216,7 @@ template <typename T>
 struct SourceAccess<PlainView<T>> {
     using View = PlainView<T>;
     static constexpr bool FLATTENS = true; // contiguous rows may be treated as one long row
+    static constexpr bool PAIRS_ROWS = false;
     template <typename O, bool SPLIT>
     static constexpr int pixels() { return pixels_per_thread<T, O, SPLIT>(); }
     template <int K>
@@ -248,6 +249,11 @@ struct SourceAccess<YuvView<PF>> {
     using Pixel = typename View::Pixel;
     using Layout = fk::detail::YuvLayout<PF>;
     static constexpr bool FLATTENS = false;
+    static constexpr bool pairs_rows() { // 4:2:0: rows 2k and 2k + 1 share a chroma row
+        if constexpr (Layout::semi_planar) return Layout::row_shift == 1;
+        else return false;
+    }
+    static constexpr bool PAIRS_ROWS = pairs_rows();
     // smallest power of two >= 4 whose output run is whole 16-byte pieces and whose luma run is whole dwords
     template <typename O, bool SPLIT>
     static constexpr int pixels() {
@@ -331,6 +337,7 @@ struct PointwiseJob {
     Out out;
     unsigned tx_shift; // log2 of the thread columns of a block; the other threads cover further rows
     unsigned grid_x, grid_y;
+    unsigned pair_limit; // blocks that are re-dealt so that row pairs share an XCD (0: none)
     size_t lds_bytes() const { return LDS_BYTES; }
 
     // A block that lies on one row and owns `span` pixels of it from pixel bx0 on (a whole number of thread groups, so
@@ -402,6 +409,19 @@ struct PointwiseJob {
         const Plane& pl = job.plane[N == 1 ? 0u : bz];
         const View& v = pl.prog.view;
         const int tid = dev::thread_in_block();
+        // pair_limit != 0 (one row per block row, the source shares a chroma row between rows 2k and 2k + 1): workgroups go
+        // to the eight XCDs round-robin in launch order, so blocks b and b + 8 run on the same XCD one after the other.
+        // Giving them the same columns of rows 2k and 2k + 1 lets the second find the chroma row in that XCD's L2 instead
+        // of fetching it from memory again through another one.  The first pair_limit blocks (a multiple of 16 and of two
+        // block rows) are dealt out that way among themselves; the few after them keep their places.
+        const unsigned launch_index = bx + job.grid_x * by;
+        if (launch_index < job.pair_limit) {
+            const unsigned xcd = launch_index & 7u, turn = launch_index >> 3;
+            const unsigned pair = 8u * (turn >> 1) + xcd; // (columns, row pair) in the order the XCDs take them up
+            const unsigned k = pair / job.grid_x;
+            bx = pair - k * job.grid_x;
+            by = 2u * k + (turn & 1u);
+        }
         const int cols = 1 << job.tx_shift;
         const int x0 = (static_cast<int>(bx) * cols + (tid & (cols - 1))) * K;
         const int y = static_cast<int>(by) * (BLOCK_THREADS >> job.tx_shift) + (tid >> job.tx_shift);
