@@ -7,6 +7,8 @@
 #include <cmath>
 #include <cstdio>
 #include <cstring>
+#include <thread>
+#include <vector>
 
 using namespace fk;
 
@@ -372,6 +374,62 @@ int main() {
             }
         }
         EXPECT(mismatches == 0);
+    }
+    // 13. executeOperations keeps no state of its own: host threads on streams of their own, each with its own buffers,
+    // launch the same chains at the same time (one small enough for by-value parameters, one batch large enough for the
+    // staged parameter block) and get what a single thread gets
+    {
+        constexpr int THREADS = 4, ROUNDS = 12;
+        constexpr size_t BATCH = 50;
+        Ptr2D<uchar3> source(640, 360);
+        fill_ramp(source, stream, 3);
+        std::array<Rect, BATCH> rects;
+        for (size_t i = 0; i < BATCH; ++i) rects[i] = Rect(static_cast<uint>(7 * i), static_cast<uint>(3 * i), 40 + 5 * static_cast<int>(i), 30 + 4 * static_cast<int>(i));
+        const auto run_batch = [&](Stream& s, Tensor<float>& out) {
+            executeOperations<TransformDPP<>>(s,
+                PerThreadRead<ND::_2D, uchar3>::build(source).then(Crop<>::build(rects)).then(Resize<InterpolationType::INTER_LINEAR>::build(Size(64, 48))),
+                Mul<float3>::build(make_set<float3>(1.f / 255.f)), TensorSplit<float3>::build(out));
+        };
+        const auto run_plain = [&](Stream& s, Ptr2D<float3>& out) {
+            executeOperations<TransformDPP<>>(s, PerThreadRead<ND::_2D, uchar3>::build(source), Cast<uchar3, float3>::build(),
+                                              Add<float3>::build(make_set<float3>(0.25f)), PerThreadWrite<ND::_2D, float3>::build(out));
+        };
+        Tensor<float> want_batch(64, 48, BATCH, 3);
+        Ptr2D<float3> want_plain(640, 360);
+        run_batch(stream, want_batch);
+        run_plain(stream, want_plain);
+        want_batch.download(stream);
+        want_plain.download(stream);
+        stream.sync();
+        int bad[THREADS] = {};
+        std::vector<std::thread> workers;
+        for (int t = 0; t < THREADS; ++t) {
+            workers.emplace_back([&, t]() {
+                try {
+                    Stream mine;
+                    Tensor<float> got_batch(64, 48, BATCH, 3);
+                    Ptr2D<float3> got_plain(640, 360);
+                    for (int round = 0; round < ROUNDS; ++round) {
+                        setTo(-1.f, got_batch, mine);
+                        run_batch(mine, got_batch);
+                        run_plain(mine, got_plain);
+                        got_batch.download(mine);
+                        got_plain.download(mine);
+                        mine.sync();
+                        if (std::memcmp(got_batch.ptrPinned().data, want_batch.ptrPinned().data, got_batch.sizeInBytes()) != 0) ++bad[t];
+                        for (uint y = 0; y < 360; y += 7)
+                            for (uint x = 0; x < 640; ++x)
+                                if (std::memcmp(&got_plain.at(x, y), &want_plain.at(x, y), sizeof(float3)) != 0) ++bad[t];
+                    }
+                } catch (const std::exception& e) {
+                    std::printf("thread %d: %s\n", t, e.what());
+                    bad[t] = -1;
+                }
+            });
+        }
+        for (auto& w : workers) w.join();
+        for (int t = 0; t < THREADS; ++t) EXPECT(bad[t] == 0);
+        EXPECT(source.getRefCount() == 1);
     }
     // 8. a launch the runtime rejects surfaces as the reference's exception text
     {
