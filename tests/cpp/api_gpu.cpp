@@ -431,6 +431,31 @@ int main() {
         for (int t = 0; t < THREADS; ++t) EXPECT(bad[t] == 0);
         EXPECT(source.getRefCount() == 1);
     }
+    // 14. a batch whose parameter block is far beyond 4 KiB and still travels by value: 200 crops in one launch against
+    // 200 launches of one crop each
+    {
+        constexpr size_t BATCH = 200;
+        Ptr2D<uchar3> source(512, 256);
+        fill_ramp(source, stream, 5);
+        std::array<Rect, BATCH> rects;
+        for (size_t i = 0; i < BATCH; ++i) rects[i] = Rect(static_cast<uint>(2 * i), static_cast<uint>(i), 20 + static_cast<int>(i % 90), 12 + static_cast<int>(i % 40));
+        Tensor<float3> together(32, 24, BATCH), one_by_one(32, 24, BATCH);
+        executeOperations<TransformDPP<>>(stream,
+            PerThreadRead<ND::_2D, uchar3>::build(source).then(Crop<>::build(rects)).then(Resize<InterpolationType::INTER_LINEAR>::build(Size(32, 24))),
+            Mul<float3>::build(make_set<float3>(0.5f)), TensorWrite<float3>::build(together));
+        for (size_t i = 0; i < BATCH; ++i) {
+            executeOperations<TransformDPP<>>(stream,
+                PerThreadRead<ND::_2D, uchar3>::build(source).then(Crop<>::build(rects[i])).then(Resize<InterpolationType::INTER_LINEAR>::build(Size(32, 24))),
+                Mul<float3>::build(make_set<float3>(0.5f)), PerThreadWrite<ND::_2D, float3>::build(one_by_one.getPlane(static_cast<uint>(i))));
+        }
+        together.download(stream);
+        one_by_one.download(stream);
+        stream.sync();
+        EXPECT(std::memcmp(together.ptrPinned().data, one_by_one.ptrPinned().data, together.sizeInBytes()) == 0);
+        bool varied = false;
+        for (uint x = 1; x < 32; ++x) varied = varied || together.at(x, 3, 150).x != together.at(0, 3, 150).x;
+        EXPECT(varied);
+    }
     // 8. a launch the runtime rejects surfaces as the reference's exception text
     {
         bool threw = false;
