@@ -44,6 +44,14 @@ __device__ __attribute__((always_inline)) inline void block_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
 }
 
+// Orders a wave's own LDS traffic: the LDS executes one wave's instructions in the order they were issued, so lanes
+// see what other lanes of the same wave wrote before this point; only the compiler has to be kept from moving them.
+__device__ __attribute__((always_inline)) inline void wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 constexpr int gcd(int a, int b) { return b == 0 ? a : gcd(b, a % b); }
 // widest transaction (16, 8 or 4 bytes) that tiles NBYTES
 constexpr int chunk_bytes(int nbytes) { return gcd(nbytes, 16); }
@@ -346,21 +354,26 @@ struct PointwiseJob {
     __device__ __attribute__((always_inline)) static inline void row_block(const PointwiseJob& job, const Plane& pl, int bx0, int span, int x0, int y,
                                                                           unsigned bz, int tid, unsigned char* lds) {
         const View& v = pl.prog.view;
-        dev::u32x4* const stage = reinterpret_cast<dev::u32x4*>(lds);
+        // A wave's 64 threads own 64*K consecutive pixels, so a wave moves its own span through its own part of the
+        // buffer and never waits for the other waves of the block.
+        const int wave = tid >> 6, lane = tid & 63;
+        dev::u32x4* const stage = reinterpret_cast<dev::u32x4*>(lds) + wave * (64 * STAGE_BYTES / 16);
         const bool active = FULL || x0 < v.w;
         Src in[K];
         if constexpr (STAGE_IN) {
-            const dev::u32x4* const g = reinterpret_cast<const dev::u32x4*>(Access::row(v, y) + static_cast<size_t>(bx0) * sizeof(Src));
-            const int pieces = span * static_cast<int>(sizeof(Src)) / 16;
+            constexpr int MINE = IN_BYTES / 16;
+            const dev::u32x4* const g =
+                reinterpret_cast<const dev::u32x4*>(Access::row(v, y) + static_cast<size_t>(bx0) * sizeof(Src)) + wave * (64 * MINE);
+            const int pieces = span * static_cast<int>(sizeof(Src)) / 16 - wave * (64 * MINE); // of this wave's span
 #pragma unroll
-            for (int j = 0; j < IN_BYTES / 16; ++j) {
-                if (FULL || j * BLOCK_THREADS + tid < pieces) stage[j * BLOCK_THREADS + tid] = g[j * BLOCK_THREADS + tid];
+            for (int j = 0; j < MINE; ++j) {
+                if (FULL || j * 64 + lane < pieces) stage[j * 64 + lane] = g[j * 64 + lane];
             }
-            dev::block_sync();
+            dev::wave_sync();
             if (active) {
-                dev::u32x4 mine[IN_BYTES / 16];
+                dev::u32x4 mine[MINE];
 #pragma unroll
-                for (int j = 0; j < IN_BYTES / 16; ++j) mine[j] = stage[tid * (IN_BYTES / 16) + j];
+                for (int j = 0; j < MINE; ++j) mine[j] = stage[lane * MINE + j];
                 __builtin_memcpy(in, mine, IN_BYTES);
             }
         } else {
@@ -372,31 +385,32 @@ struct PointwiseJob {
             for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
         }
         if constexpr (STAGE_OUT) {
-            if constexpr (STAGE_IN) dev::block_sync(); // every thread has taken its input out of the buffer
+            constexpr int MINE = OUT_BYTES / 16;
+            if constexpr (STAGE_IN) dev::wave_sync(); // every lane has taken its input out of the buffer
             if (active) {
                 unsigned int w[OUT_BYTES / 4];
                 dev::pack_pixels<K>(o, w);
 #pragma unroll
-                for (int j = 0; j < OUT_BYTES / 16; ++j) {
+                for (int j = 0; j < MINE; ++j) {
                     dev::u32x4 piece;
                     piece.x = w[4 * j]; piece.y = w[4 * j + 1]; piece.z = w[4 * j + 2]; piece.w = w[4 * j + 3];
-                    stage[tid * (OUT_BYTES / 16) + j] = piece;
+                    stage[lane * MINE + j] = piece;
                 }
             }
-            dev::block_sync();
+            dev::wave_sync();
             dev::u32x4* const g = reinterpret_cast<dev::u32x4*>(
                 reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
-                static_cast<size_t>(y) * job.out.pitch + static_cast<size_t>(bx0) * sizeof(OutPixel));
-            const int pieces = span * static_cast<int>(sizeof(OutPixel)) / 16;
+                static_cast<size_t>(y) * job.out.pitch + static_cast<size_t>(bx0) * sizeof(OutPixel)) + wave * (64 * MINE);
+            const int pieces = span * static_cast<int>(sizeof(OutPixel)) / 16 - wave * (64 * MINE);
             if ((pl.flags & FLAG_STREAM_STORES) != 0u) {
 #pragma unroll
-                for (int j = 0; j < OUT_BYTES / 16; ++j) {
-                    if (FULL || j * BLOCK_THREADS + tid < pieces) dev::store_piece<true>(g + j * BLOCK_THREADS + tid, stage[j * BLOCK_THREADS + tid]);
+                for (int j = 0; j < MINE; ++j) {
+                    if (FULL || j * 64 + lane < pieces) dev::store_piece<true>(g + j * 64 + lane, stage[j * 64 + lane]);
                 }
             } else {
 #pragma unroll
-                for (int j = 0; j < OUT_BYTES / 16; ++j) {
-                    if (FULL || j * BLOCK_THREADS + tid < pieces) g[j * BLOCK_THREADS + tid] = stage[j * BLOCK_THREADS + tid];
+                for (int j = 0; j < MINE; ++j) {
+                    if (FULL || j * 64 + lane < pieces) g[j * 64 + lane] = stage[j * 64 + lane];
                 }
             }
         } else if (active) {
