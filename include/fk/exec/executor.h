@@ -175,6 +175,14 @@ struct JobOf {
             job.active = sender.getActiveThreads();
             job.grid_x = job.plan(job.active);
             job.grid_y = ceil_div(job.active.y, 4u);
+            job.packs_rows = 0u;
+            if constexpr (decltype(job)::PACKS_ROWS) {
+                const auto out = OutOf<Receiver>::make(receiver);
+                job.packs_rows = (aligned_to(out.data, 4) && out.pitch % 4u == 0u && out.z_stride % 4u == 0u) ? 1u : 0u;
+                job.out_data = reinterpret_cast<char*>(out.data);
+                job.out_pitch = out.pitch;
+                job.out_z_stride = out.z_stride;
+            }
             return job;
         }
     }

@@ -773,6 +773,20 @@ struct GenericJob {
     ActiveThreads active;
     unsigned grid_x, grid_y;
     unsigned wide; // 4 elements per thread instead of 1
+    // A packed receiver whose pixels are not whole dwords (three bytes, say) would be written with byte stores.  With
+    // four elements per thread such a job gives a thread four neighbouring pixels instead of four that are 64 apart:
+    // they are sizeof(pixel) whole dwords of the row, packed in registers and stored at once.
+    using OutView = OutOf<Receiver>;
+    template <typename V, typename = void>
+    struct PacksRows : std::false_type {};
+    template <typename V>
+    struct PacksRows<V, std::enable_if_t<V::supported>>
+        : std::bool_constant<!V::type::IS_SPLIT && sizeof(typename V::type::Pixel) % 4 != 0 && std::is_same_v<typename V::type::Pixel, Value>> {};
+    static constexpr bool PACKS_ROWS = PacksRows<OutView>::value;
+    unsigned packs_rows; // the receiver's rows start at whole dwords (decided by the host, which then also fills in:)
+    char* out_data;      // element (0, 0, 0) of the receiver, bytes between its rows and between its planes
+    unsigned out_pitch;
+    size_t out_z_stride;
     size_t lds_bytes() const { return 0; }
     // decides the elements per thread from the size of the output and returns the number of blocks along x
     unsigned plan(const ActiveThreads& extent) {
@@ -785,9 +799,35 @@ struct GenericJob {
     template <int K>
     __device__ __attribute__((always_inline)) static inline void body(const GenericJob& job, unsigned bx, unsigned by, unsigned bz) {
         const int tid = dev::thread_in_block();
-        const int x0 = static_cast<int>(bx) * (64 * K) + (tid & 63);
         const int y = static_cast<int>(by) * 4 + (tid >> 6);
         const int w = static_cast<int>(job.active.x);
+        if constexpr (PACKS_ROWS && K == 4) {
+            if (job.packs_rows != 0u) {
+                const int x0 = static_cast<int>(bx) * (64 * K) + (tid & 63) * K;
+                if (x0 >= w || y >= static_cast<int>(job.active.y)) return;
+                Value value[K];
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    const int x = x0 + k < w ? x0 + k : w - 1;
+                    value[k] = Sender::Operation::exec(Point(x, y, static_cast<int>(bz)), job.sender);
+                }
+                if (x0 + K <= w) {
+                    constexpr int S = static_cast<int>(sizeof(Value)); // bytes per pixel = dwords per thread
+                    unsigned int words[S];
+                    dev::pack_pixels<K>(value, words);
+                    char* const run = job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch +
+                                      static_cast<size_t>(x0) * S;
+                    __builtin_memcpy(__builtin_assume_aligned(run, 4), words, 4 * S);
+                } else {
+#pragma unroll
+                    for (int k = 0; k < K; ++k) {
+                        if (x0 + k < w) Receiver::Operation::exec(Point(x0 + k, y, static_cast<int>(bz)), value[k], job.receiver);
+                    }
+                }
+                return;
+            }
+        }
+        const int x0 = static_cast<int>(bx) * (64 * K) + (tid & 63);
         if (x0 >= w || y >= static_cast<int>(job.active.y)) return;
         Value value[K];
 #pragma unroll

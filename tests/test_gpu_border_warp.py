@@ -137,6 +137,14 @@ def test_large_outputs_vs_oracle(fk, oracle):
     fk.border_crop_u8c3(B.BORDER_REFLECT, d_src, 300, 300, big)
     torch.cuda.synchronize()
     assert same_bits(host(big), oracle.border_crop_u8c3(B.BORDER_REFLECT, src, 300, 300, (w + 600, h + 600)))
+    # rows that start at whole dwords (2532 * 3 bytes): a thread then packs four neighbouring pixels into three dwords;
+    # the width is odd, so the last thread of a row holds one pixel
+    for bt in (B.BORDER_REFLECT_101, B.BORDER_WRAP, B.BORDER_CONSTANT):
+        packed = out_u8(w + 601, h + 600, 1)
+        fk.border_crop_u8c3(bt, d_src, 300, 300, packed)
+        torch.cuda.synchronize()
+        assert same_bits(host(packed), oracle.border_crop_u8c3(bt, src, 300, 300, (w + 601, h + 600))), bt
+        assert bool((packed._base[:, w + 601:] == 85).all()), "the padding of the rows was written"
 
 
 def test_argument_errors(fk):
