@@ -775,7 +775,8 @@ struct GenericJob {
     unsigned wide; // 4 elements per thread instead of 1
     // A packed receiver whose pixels are not whole dwords (three bytes, say) would be written with byte stores.  With
     // four elements per thread such a job gives a thread four neighbouring pixels instead of four that are 64 apart:
-    // they are sizeof(pixel) whole dwords of the row, packed in registers and stored at once.
+    // they are sizeof(pixel) whole dwords of the row, packed in registers and stored at once.  (For every other job
+    // neighbours are the slower choice: each memory instruction of a wave then covers a quarter of the lines' bytes.)
     using OutView = OutOf<Receiver>;
     template <typename V, typename = void>
     struct PacksRows : std::false_type {};
@@ -796,53 +797,46 @@ struct GenericJob {
         return (extent.x + tile_w - 1u) / tile_w;
     }
 
-    template <int K>
+    // K elements per thread: NEIGHBOURS, or 64 apart (then each of a wave's memory instructions covers 64 neighbours).
+    template <int K, bool NEIGHBOURS>
     __device__ __attribute__((always_inline)) static inline void body(const GenericJob& job, unsigned bx, unsigned by, unsigned bz) {
+        constexpr int STEP = NEIGHBOURS ? 1 : 64;
         const int tid = dev::thread_in_block();
         const int y = static_cast<int>(by) * 4 + (tid >> 6);
         const int w = static_cast<int>(job.active.x);
-        if constexpr (PACKS_ROWS && K == 4) {
-            if (job.packs_rows != 0u) {
-                const int x0 = static_cast<int>(bx) * (64 * K) + (tid & 63) * K;
-                if (x0 >= w || y >= static_cast<int>(job.active.y)) return;
-                Value value[K];
-#pragma unroll
-                for (int k = 0; k < K; ++k) {
-                    const int x = x0 + k < w ? x0 + k : w - 1;
-                    value[k] = Sender::Operation::exec(Point(x, y, static_cast<int>(bz)), job.sender);
-                }
-                if (x0 + K <= w) {
-                    constexpr int S = static_cast<int>(sizeof(Value)); // bytes per pixel = dwords per thread
-                    unsigned int words[S];
-                    dev::pack_pixels<K>(value, words);
-                    char* const run = job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch +
-                                      static_cast<size_t>(x0) * S;
-                    __builtin_memcpy(__builtin_assume_aligned(run, 4), words, 4 * S);
-                } else {
-#pragma unroll
-                    for (int k = 0; k < K; ++k) {
-                        if (x0 + k < w) Receiver::Operation::exec(Point(x0 + k, y, static_cast<int>(bz)), value[k], job.receiver);
-                    }
-                }
-                return;
-            }
-        }
-        const int x0 = static_cast<int>(bx) * (64 * K) + (tid & 63);
+        const int x0 = static_cast<int>(bx) * (64 * K) + (tid & 63) * (NEIGHBOURS ? K : 1);
         if (x0 >= w || y >= static_cast<int>(job.active.y)) return;
         Value value[K];
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            const int x = x0 + 64 * k < w ? x0 + 64 * k : w - 1;
+            const int x = x0 + STEP * k < w ? x0 + STEP * k : w - 1;
             value[k] = Sender::Operation::exec(Point(x, y, static_cast<int>(bz)), job.sender);
+        }
+        if constexpr (PACKS_ROWS && NEIGHBOURS && K == 4) {
+            if (job.packs_rows != 0u && x0 + K <= w) {
+                constexpr int S = static_cast<int>(sizeof(Value)); // bytes per pixel = dwords per thread
+                unsigned int words[S];
+                dev::pack_pixels<K>(value, words);
+                char* const run = job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch +
+                                  static_cast<size_t>(x0) * S;
+                __builtin_memcpy(__builtin_assume_aligned(run, 4), words, 4 * S);
+                return;
+            }
         }
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            if (x0 + 64 * k < w) Receiver::Operation::exec(Point(x0 + 64 * k, y, static_cast<int>(bz)), value[k], job.receiver);
+            if (x0 + STEP * k < w) Receiver::Operation::exec(Point(x0 + STEP * k, y, static_cast<int>(bz)), value[k], job.receiver);
         }
     }
     __device__ __attribute__((always_inline)) static inline void run(const GenericJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char*) {
-        if (job.wide != 0u) body<4>(job, bx, by, bz);
-        else body<1>(job, bx, by, bz);
+        if constexpr (PACKS_ROWS) { // the only jobs that are compiled with the neighbour form
+            if (job.wide != 0u && job.packs_rows != 0u) {
+                body<4, true>(job, bx, by, bz);
+                return;
+            }
+        }
+        if (job.wide != 0u) body<4, false>(job, bx, by, bz);
+        else body<1, false>(job, bx, by, bz);
     }
 };
 

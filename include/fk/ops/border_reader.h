@@ -87,10 +87,12 @@ public:
         const int width = static_cast<int>(BackIOp::Operation::num_elems_x(thread, backIOp));
         const int height = static_cast<int>(BackIOp::Operation::num_elems_y(thread, backIOp));
         if constexpr (BT == BorderType::CONSTANT) {
-            if (thread.x >= 0 && thread.x < width && thread.y >= 0 && thread.y < height) {
-                return BackIOp::Operation::exec(thread, backIOp);
-            }
-            return params.value;
+            // No branch around the read: a coordinate outside reads element (0, 0) and drops it.  A thread that handles
+            // several elements can then have all its reads in flight at once instead of waiting for each in turn.
+            const bool inside = thread.x >= 0 && thread.x < width && thread.y >= 0 && thread.y < height;
+            const Point source(inside ? thread.x : 0, inside ? thread.y : 0, thread.z);
+            const OutputType sample = BackIOp::Operation::exec(source, backIOp);
+            return inside ? sample : params.value;
         } else {
             const Point source(detail::border_index<BT>(thread.x, width), detail::border_index<BT>(thread.y, height), thread.z);
             return BackIOp::Operation::exec(source, backIOp);
