@@ -107,7 +107,14 @@ public:
             // (the limits are integers, so rounding leaves them alone), then round half away from zero through int.
             const I above = static_cast<I>(hi), below = static_cast<I>(lo);
             I clamped{};
-            if constexpr (std::is_same_v<I, float>) clamped = __builtin_fmaxf(__builtin_fminf(input, above), below);
+            if constexpr (std::is_same_v<I, float>) {
+#if defined(__HIP_DEVICE_COMPILE__)
+                // the median of (input, lowest, highest) is the clamped value, in one instruction
+                if (!__builtin_is_constant_evaluated()) clamped = __builtin_amdgcn_fmed3f(input, below, above);
+                else
+#endif
+                    clamped = __builtin_fmaxf(__builtin_fminf(input, above), below);
+            }
             else clamped = static_cast<I>(__builtin_fmax(__builtin_fmin(static_cast<double>(input), static_cast<double>(above)), static_cast<double>(below)));
             if constexpr (std::is_unsigned_v<O>) {
                 return static_cast<O>(static_cast<int>(clamped + I(0.5))); // clamped >= 0, and (int)(0 - 0.5) == (int)(0 + 0.5)

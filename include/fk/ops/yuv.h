@@ -278,6 +278,26 @@ private:
     static_assert(cn<Packed> == 3, "ConvertYUVToRGB takes three-channel YUV pixels");
     static_assert(cn<ReturnType> == (ALPHA ? 4 : 3), "ReturnType must have 4 channels with ALPHA, 3 without");
 
+    // MxVFloat3 on a centred pixel with the matrix as compile-time constants, without the terms whose coefficient is
+    // zero (two of the nine in every YCbCr -> RGB matrix).  The results are the same bits: the chroma differences are
+    // finite, so such a term is +0 or -0, and the sum it would be added to is never -0 (luma comes from an integer, and
+    // x - x is +0), so adding it changes nothing.
+    static constexpr M3x3Float MATRIX = ccMatrix<CR, CP, ColorConversionDir::YCbCr2RGB>;
+    template <int ROW>
+    static constexpr float3 matrix_row() {
+        if constexpr (ROW == 0) return MATRIX.x;
+        else if constexpr (ROW == 1) return MATRIX.y;
+        else return MATRIX.z;
+    }
+    template <int ROW>
+    FK_HD_STATIC float row_times(const float3& v) {
+        constexpr float3 row = matrix_row<ROW>();
+        float sum = v.x * row.x;
+        if constexpr (row.y != 0.f) sum = sum + v.y * row.y;
+        if constexpr (row.z != 0.f) sum = sum + v.z * row.z;
+        return sum;
+    }
+
 public:
     static constexpr ColorDepth CD = PixelFormatTraits<PF>::depth;
     FK_UNARY_OPERATION(ConvertYUVToRGB, Packed, ReturnType)
@@ -289,7 +309,7 @@ public:
         constexpr float lumaSub = CP == ColorPrimitives::bt601 ? subCoefficients<CD>.luma : 0.f;
         float3 centred{ static_cast<float>(yuv.x), yuv.y - chromaSub, yuv.z - chromaSub };
         if constexpr (CP == ColorPrimitives::bt601) centred.x = yuv.x - lumaSub;
-        const float3 rgb = MxVFloat3<>::exec(centred, ccMatrix<CR, CP, ColorConversionDir::YCbCr2RGB>);
+        const float3 rgb{ row_times<0>(centred), row_times<1>(centred), row_times<2>(centred) };
         if constexpr (std::is_same_v<VBase<OutputType>, float>) {
             constexpr float scale = floatShiftFactor<CD>;
             if constexpr (ALPHA) {
