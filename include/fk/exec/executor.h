@@ -112,11 +112,9 @@ struct JobOf {
                 if constexpr (Out::IS_SPLIT) vec = vec && out.chan_stride % 16 == 0;
                 const bool stream = static_cast<size_t>(max_w) * max_h * N * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
                 job.flags = (vec ? FLAG_VECTOR_IO : 0u) | (vec && stream ? FLAG_STREAM_STORES : 0u);
-                for (size_t i = 0; i < N; ++i) {
-                    if (decltype(job)::worth_staging(job.plane[i].view.fx, job.plane[i].view.fy)) job.flags |= FLAG_SOURCE_TILE;
-                }
                 // small outputs gain nothing from leaving through LDS, and the LDS they would ask for lowers occupancy
                 if (vec && static_cast<size_t>(max_w) * max_h * N * sizeof(typename Out::Pixel) >= (1u << 20)) job.flags |= FLAG_STAGE_OUT;
+                job.plan_lds(); // sets FLAG_SOURCE_TILE when some plane's tiles are worth staging
                 return job;
             } else {
                 using Job = PointwiseJob<Prog, N, Out>;

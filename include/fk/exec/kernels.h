@@ -554,16 +554,36 @@ struct ResizeJob {
     // tiles are worth staging in LDS; FLAG_STAGE_OUT: packed output leaves through LDS.  The last two decide how much
     // LDS the launch asks for (a divergent launch shares one LDS size between all its jobs).
     unsigned flags;
+    // The launch asks for as much LDS as the planes' own factors need, not for the capacity: a block's LDS decides how
+    // many blocks a CU holds.  tile_dwords is the room for a source tile (a tile that needs more reads its taps
+    // directly); the packed output is staged behind it when both fit the capacity (out_stage_offset, in bytes), else in
+    // the same place (0), which costs a block barrier between the last tap and the first staged pixel.
+    unsigned tile_dwords;
+    unsigned out_stage_offset;
     size_t lds_bytes() const {
         size_t n = 0;
-        if ((flags & FLAG_SOURCE_TILE) != 0u) n = RESIZE_LDS_DWORDS * 4;
-        if (STAGE_OUT && (flags & FLAG_STAGE_OUT) != 0u && static_cast<size_t>(OUT_STAGE_BYTES) > n) n = OUT_STAGE_BYTES;
+        if ((flags & FLAG_SOURCE_TILE) != 0u) n = static_cast<size_t>(tile_dwords) * 4;
+        if (STAGE_OUT && (flags & FLAG_STAGE_OUT) != 0u && out_stage_offset + static_cast<size_t>(OUT_STAGE_BYTES) > n) n = out_stage_offset + OUT_STAGE_BYTES;
         return n == 0 ? 0 : n + 16;
     }
-    // whether a tile of a plane with these factors can be staged (same rule as the kernel applies per tile)
-    static bool worth_staging(float fx, float fy) {
+    // dwords a tile of a plane with these factors takes when staged, 0 when it is not worth staging (same rule as the
+    // kernel applies per tile)
+    static unsigned staged_tile_dwords(float fx, float fy) {
         const int cols = static_cast<int>((RESIZE_TILE_W - 1) * fx) + 3, rows = static_cast<int>((RESIZE_TILE_H - 1) * fy) + 3;
-        return rows * (cols | 1) * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * RESIZE_TILE_W * RESIZE_TILE_H + 256;
+        const bool worth = rows * (cols | 1) * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * RESIZE_TILE_W * RESIZE_TILE_H + 256;
+        return worth ? static_cast<unsigned>(rows * (cols | 1) * SLOT) : 0u;
+    }
+    // fills in the LDS layout from the planes' factors; FLAG_STAGE_OUT has been decided
+    void plan_lds() {
+        tile_dwords = 0;
+        for (size_t i = 0; i < N; ++i) {
+            const unsigned need = staged_tile_dwords(plane[i].view.fx, plane[i].view.fy);
+            tile_dwords = need > tile_dwords ? need : tile_dwords;
+        }
+        tile_dwords = (tile_dwords + 3u) & ~3u; // what follows the tile starts at a whole 16 bytes
+        if (tile_dwords != 0u) flags |= FLAG_SOURCE_TILE;
+        const bool behind = STAGE_OUT && (flags & FLAG_STAGE_OUT) != 0u && tile_dwords * 4u + OUT_STAGE_BYTES <= RESIZE_LDS_DWORDS * 4u;
+        out_stage_offset = behind ? tile_dwords * 4u : 0u;
     }
 
     // source pixel (x, y) of the resampled window, after the operations fused before the resize
@@ -668,7 +688,7 @@ struct ResizeJob {
             stride = cols | 1;
             const int tile_px = (rx_hi - rx_lo + 1) * (ry_hi - ry_lo + 1);
             // staging pays off while a source pixel is used about once or more; strong down-scaling reads taps directly
-            staged = (job.flags & FLAG_SOURCE_TILE) != 0u && rows * stride * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * tile_px + 256;
+            staged = (job.flags & FLAG_SOURCE_TILE) != 0u && rows * stride * SLOT <= static_cast<int>(job.tile_dwords) && rows * cols <= 3 * tile_px + 256;
             if (staged) {
                 const int wave = tid >> 6, lane = tid & 63;
                 for (int r = wave; r < rows; r += BLOCK_THREADS / 64) {
@@ -720,20 +740,24 @@ struct ResizeJob {
             if (whole_width && (job.flags & FLAG_STAGE_OUT) != 0u) {
                 constexpr int PIECES_PER_ROW = OUT_ROW_BYTES / 16;
                 constexpr int MINE = RESIZE_PX * static_cast<int>(sizeof(OutPixel)) / 16;
-                dev::u32x4* const stage = reinterpret_cast<dev::u32x4*>(lds_raw);
-                dev::block_sync(); // every thread is done with the source tile
+                dev::u32x4* const stage = reinterpret_cast<dev::u32x4*>(lds_raw + job.out_stage_offset);
+                // the buffer held the source tile: every thread is done with it
+                if (job.out_stage_offset == 0u && (job.flags & FLAG_SOURCE_TILE) != 0u) dev::block_sync();
+                // A wave's 64 threads own four whole rows of the tile (64 * MINE pieces), so a wave moves its rows
+                // through its own part of the buffer and never waits for the other waves of the block.
                 dev::u32x4 mine[MINE];
                 __builtin_memcpy(mine, o, sizeof(mine));
 #pragma unroll
                 for (int j = 0; j < MINE; ++j) stage[tid * MINE + j] = mine[j];
-                dev::block_sync();
+                dev::wave_sync();
+                const int wave_first = (tid >> 6) * (64 * MINE), lane = tid & 63;
                 char* const obase = reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
                                     static_cast<size_t>(ty0) * job.out.pitch + static_cast<size_t>(tx0) * sizeof(OutPixel);
                 const int rows_here = v.h - ty0 < RESIZE_TILE_H ? v.h - ty0 : RESIZE_TILE_H;
                 const bool stream = (job.flags & FLAG_STREAM_STORES) != 0u;
 #pragma unroll
-                for (int j = 0; j < RESIZE_TILE_H * PIECES_PER_ROW / BLOCK_THREADS; ++j) {
-                    const int id = j * BLOCK_THREADS + tid;
+                for (int j = 0; j < MINE; ++j) {
+                    const int id = wave_first + j * 64 + lane;
                     const int r = id / PIECES_PER_ROW, c = id - r * PIECES_PER_ROW;
                     if (r < rows_here) {
                         dev::u32x4* const g = reinterpret_cast<dev::u32x4*>(obase + static_cast<size_t>(r) * job.out.pitch) + c;
