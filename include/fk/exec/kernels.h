@@ -113,10 +113,69 @@ __device__ __attribute__((always_inline)) inline void store_words(void* p, const
     }
 }
 
+// x / d with the host's r = RN(1 / d): the short form where every lane of the wave holds an x in [2^-60, 2^60], the
+// division instruction sequence elsewhere (the branch is wave-uniform).
+template <typename F>
+__device__ __attribute__((always_inline)) inline F prepared_divide(const F& x, const F& d, const float* r, const bool fast) {
+    if (fast) {
+        float lo = __builtin_fabsf(vectorAt(0, x)), hi = lo;
+#pragma unroll
+        for (int c = 1; c < cn<F>; ++c) {
+            const float a = __builtin_fabsf(vectorAt(c, x));
+            lo = __builtin_fminf(lo, a);
+            hi = __builtin_fmaxf(hi, a);
+        }
+        // lanes inside the range (a NaN is not); each ballot is one compare, the rest is scalar work
+        const unsigned long long inside = __builtin_amdgcn_ballot_w64(lo >= PREPARED_DIV_LO) & __builtin_amdgcn_ballot_w64(hi <= PREPARED_DIV_HI);
+        if (inside == __builtin_amdgcn_ballot_w64(true)) {
+            float q[cn<F>];
+#pragma unroll
+            for (int c = 0; c < cn<F>; ++c) {
+                const float xc = vectorAt(c, x), dc = vectorAt(c, d), rc = r[c];
+                float qc = xc * rc;
+                qc = __builtin_fmaf(__builtin_fmaf(-dc, qc, xc), rc, qc);
+                qc = __builtin_fmaf(__builtin_fmaf(-dc, qc, xc), rc, qc);
+                q[c] = qc;
+            }
+            F out;
+            __builtin_memcpy(&out, q, sizeof(F));
+            return out;
+        }
+    }
+    return x / d;
+}
+
+template <int I, typename V, typename Prepared, typename Op, typename... Rest_>
+__device__ __attribute__((always_inline)) inline auto compute_prepared(const V& v, const Prepared& tail, const OperationTuple<Op, Rest_...>& t) {
+    using Tuple = OperationTuple<Op, Rest_...>;
+    constexpr bool IS_DIV = IsFloatDiv<Op>::value;
+    const auto step = [&] {
+        if constexpr (IS_DIV && std::is_same_v<V, typename Op::InputType>) {
+            return prepared_divide(v, t.instance.params, tail.recip[I], (tail.fast >> I & 1u) != 0u);
+        } else {
+            return fk::detail::chain_step<Op>(Point(), v, t);
+        }
+    }();
+    if constexpr (sizeof...(Rest_) == 0) {
+        return step;
+    } else if constexpr (Tuple::HAS_NEXT) {
+        return compute_prepared<I + (IS_DIV ? 1 : 0)>(step, tail, t.next);
+    } else {
+        return compute_prepared<I + (IS_DIV ? 1 : 0)>(step, tail, OperationTuple<Rest_...>{});
+    }
+}
+
+template <typename Tail>
+struct IsPreparedTail : std::false_type {};
+template <typename Ops, int NDIV>
+struct IsPreparedTail<PreparedTail<Ops, NDIV>> : std::true_type {};
+
 template <typename Tail, typename V>
 __device__ __attribute__((always_inline)) inline auto apply_tail(const Tail& tail, const V& v) {
     if constexpr (std::is_same_v<Tail, NoTail>) {
         return v;
+    } else if constexpr (IsPreparedTail<Tail>::value) {
+        return compute_prepared<0>(v, tail, tail.ops);
     } else {
         return fk::detail::tuple_compute(v, tail);
     }
@@ -601,6 +660,10 @@ struct ResizeJob {
         bool row_inside = INTERIOR || y < v.h;
         if constexpr (View::HAS_ROI && !INTERIOR) row_inside = row_inside && ry >= v.y1 && ry <= v.y2;
         const float src_y = (ry - v.y1) * v.fy;
+        // a short tail is taken into registers once, ahead of the pixels (read in place it is fetched where it is used,
+        // once per pixel and with the wait in the middle of the arithmetic)
+        using Tail = std::decay_t<decltype(prog.tail)>;
+        const std::conditional_t<(sizeof(Tail) <= 128), Tail, const Tail&> tail = prog.tail;
 #pragma unroll
         for (int k = 0; k < RESIZE_PX; ++k) {
             const int x = x_first + k;
@@ -643,7 +706,7 @@ struct ResizeJob {
                 }
                 value = fk::detail::bilinear_blend(a, b, c, d, t);
             }
-            o[k] = dev::apply_tail(prog.tail, value);
+            o[k] = dev::apply_tail(tail, value);
         }
     }
 

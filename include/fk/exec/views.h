@@ -72,6 +72,56 @@ struct PlaneProgram {
     Tail tail;
 };
 
+// ---- divisions by a divisor the host has seen ------------------------------------------------------------------------
+// A Div<float..> of a chain's tail divides every pixel by the same values.  IEEE division is eleven instructions on
+// this part; with r = RN(1 / d) from the host, q = x * r followed by two corrections q += fma(-d, q, x) * r is the
+// correctly rounded x / d as well (after the first correction q is RN(x / d + t) with |t| < 2^-23 ulp, hence a faithful
+// rounding; a correction of a faithful quotient by a correctly rounded reciprocal gives the correctly rounded quotient:
+// Markstein, "Computation of elementary functions on the IBM RISC System/6000 processor", 1990), as long as nothing on
+// the way leaves the normal range.  The host vouches for d (finite, 2^-60 <= |d| <= 2^60), the kernel tests x and takes
+// the division instruction sequence where a lane is outside (zeros, subnormals, infinities, huge values).
+template <typename Op>
+struct IsFloatDiv : std::false_type {};
+template <typename F>
+struct IsFloatDiv<Div<F, F, F>> : std::bool_constant<std::is_same_v<VBase<F>, float>> {};
+template <typename... Ops>
+constexpr int float_div_count = (0 + ... + (IsFloatDiv<Ops>::value ? 1 : 0));
+
+constexpr float PREPARED_DIV_LO = 8.67361738e-19f; // 2^-60
+constexpr float PREPARED_DIV_HI = 1.15292150e+18f; // 2^60
+
+template <typename Ops, int NDIV>
+struct PreparedTail {
+    Ops ops;
+    float recip[NDIV][4]; // per float division of the tail, in order: RN(1 / d) per channel
+    unsigned fast;        // bit i: every divisor of division i is in range, so its reciprocals are valid
+};
+
+namespace detail {
+inline bool prepared_divisor_ok(const float d) {
+    const float a = d < 0.f ? -d : d;
+    return a >= PREPARED_DIV_LO && a <= PREPARED_DIV_HI; // false for NaN
+}
+template <int I, typename Prepared, typename Op, typename... Rest_>
+inline void prepare_divisions(Prepared& out, const OperationTuple<Op, Rest_...>& t) {
+    constexpr bool IS_DIV = IsFloatDiv<Op>::value;
+    if constexpr (IS_DIV) {
+        using F = typename Op::ParamsType;
+        bool ok = true;
+        for (int c = 0; c < 4; ++c) out.recip[I][c] = 0.f;
+        for (int c = 0; c < cn<F>; ++c) {
+            const volatile float d = vectorAt(c, t.instance.params); // volatile: a division at run time, correctly rounded
+            ok = ok && prepared_divisor_ok(d);
+            out.recip[I][c] = ok ? 1.0f / d : 0.f;
+        }
+        if (ok) out.fast |= 1u << I;
+    }
+    if constexpr (sizeof...(Rest_) > 0) {
+        prepare_divisions<I + (IS_DIV ? 1 : 0)>(out, fk::detail::tuple_tail(t));
+    }
+}
+} // namespace detail
+
 // ---- read side ---------------------------------------------------------------------------------------------------
 template <typename IOp, typename = void>
 struct ViewOf {
@@ -230,11 +280,19 @@ struct ProgramOf<Read<FusedOperation<Head, ComputeOps...>>,
     static constexpr bool supported = true;
     using IOp = Read<FusedOperation<Head, ComputeOps...>>;
     using View = typename ViewOf<Instantiable<Head>>::type;
-    using Tail = OperationTuple<ComputeOps...>;
+    using Ops = OperationTuple<ComputeOps...>;
+    static constexpr int NDIV = float_div_count<ComputeOps...>;
+    using Tail = std::conditional_t<(NDIV > 0 && NDIV <= 32), PreparedTail<Ops, NDIV>, Ops>;
     using type = PlaneProgram<View, Tail>;
     using OutputType = typename IOp::Operation::OutputType;
     static type make(const IOp& iOp) {
-        return type{ ViewOf<Instantiable<Head>>::make(toIOp<Head>(iOp.params.instance)), fk::detail::tuple_tail(iOp.params) };
+        if constexpr (std::is_same_v<Tail, Ops>) {
+            return type{ ViewOf<Instantiable<Head>>::make(toIOp<Head>(iOp.params.instance)), fk::detail::tuple_tail(iOp.params) };
+        } else {
+            type prog{ ViewOf<Instantiable<Head>>::make(toIOp<Head>(iOp.params.instance)), Tail{ fk::detail::tuple_tail(iOp.params), {}, 0u } };
+            detail::prepare_divisions<0>(prog.tail, prog.tail.ops);
+            return prog;
+        }
     }
 };
 
