@@ -563,6 +563,15 @@ __device__ __attribute__((always_inline)) inline PixelSlot<T> load_pixel_slot(co
         const unsigned int* const p = reinterpret_cast<const unsigned int*>(row + off);
 #pragma unroll
         for (int i = 0; i < ND; ++i) s.w[i] = p[i];
+    } else if constexpr (sizeof(T) == 3) {
+        // one unaligned dword, [p, p + 4) for an aligned p and [p - 1, p + 3) otherwise: its one byte that is not the
+        // pixel's lies in an aligned dword that also holds a byte of the pixel, so the load cannot fault and needs no
+        // branch (the loads of several rows are in flight together)
+        const char* const p = row + off;
+        const unsigned back = (static_cast<unsigned>(reinterpret_cast<size_t>(p)) & 3u) != 0u ? 1u : 0u;
+        unsigned int w;
+        __builtin_memcpy(&w, p - back, 4);
+        s.w[0] = w >> (8u * back);
     } else {
         const unsigned mis = (static_cast<unsigned>(reinterpret_cast<size_t>(row)) + static_cast<unsigned>(off)) & 3u;
         const int first = off - static_cast<int>(mis); // aligned dword that holds the pixel's first byte
@@ -664,6 +673,8 @@ struct ResizeJob {
         // once per pixel and with the wait in the middle of the arithmetic)
         using Tail = std::decay_t<decltype(prog.tail)>;
         const std::conditional_t<(sizeof(Tail) <= 128), Tail, const Tail&> tail = prog.tail;
+        // the float of (rx - x1) for the thread's first pixel; the next ones are that plus 1, 2, 3 (exact: far below 2^24)
+        const float rel_x0 = static_cast<float>(x_first + v.off_x - v.x1);
 #pragma unroll
         for (int k = 0; k < RESIZE_PX; ++k) {
             const int x = x_first + k;
@@ -672,7 +683,7 @@ struct ResizeJob {
             if constexpr (View::HAS_ROI && !INTERIOR) inside = inside && rx >= v.x1 && rx <= v.x2;
             Pixel value = v.background;
             if (inside) {
-                const float src_x = (rx - v.x1) * v.fx;
+                const float src_x = (rel_x0 + static_cast<float>(k)) * v.fx;
                 const fk::detail::BilinearTaps t = fk::detail::bilinear_taps(src_x, src_y, Size(s.w, s.h));
                 Src a, b, c, d;
                 if constexpr (STAGED) {
@@ -753,23 +764,37 @@ struct ResizeJob {
             // staging pays off while a source pixel is used about once or more; strong down-scaling reads taps directly
             staged = (job.flags & FLAG_SOURCE_TILE) != 0u && rows * stride * SLOT <= static_cast<int>(job.tile_dwords) && rows * cols <= 3 * tile_px + 256;
             if (staged) {
-                const int wave = tid >> 6, lane = tid & 63;
-                for (int r = wave; r < rows; r += BLOCK_THREADS / 64) {
-                    const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
-                    const char* const row = window + static_cast<size_t>(sy) * s.pitch;
-                    for (int c = lane; c < cols; c += 64) {
-                        const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
-                        dev::PixelSlot<Src> px;
-                        if constexpr (RAW_SOURCE) {
-                            px = dev::load_pixel_slot<Src>(row, sx * static_cast<int>(sizeof(Src)), valid_lo, valid_hi);
-                        } else {
-                            const Src value = fetch(v, sx, sy);
+                // A wave takes every fourth row, a lane every 64th column; the loads of STAGE_ROWS rows are issued before
+                // the first of them is stored, so a tile of up to 4 * STAGE_ROWS rows costs one memory round trip.  A row
+                // past the tile's last is the last one again, loaded and stored twice: with a branch around it the
+                // compiler moves the load to the store and waits there.
+                const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+                constexpr int WAVES = BLOCK_THREADS / 64;
+                constexpr int STAGE_ROWS = SLOT == 1 ? 4 : 2;
+                for (int c = lane; c < cols; c += 64) {
+                    const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
+                    for (int r0 = wave; r0 < rows; r0 += WAVES * STAGE_ROWS) {
+                        dev::PixelSlot<Src> px[STAGE_ROWS];
 #pragma unroll
-                            for (int i = 0; i < SLOT; ++i) px.w[i] = 0u;
-                            __builtin_memcpy(px.w, &value, sizeof(Src));
+                        for (int u = 0; u < STAGE_ROWS; ++u) {
+                            const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
+                            const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
+                            if constexpr (RAW_SOURCE) {
+                                const char* const row = window + static_cast<size_t>(sy) * s.pitch;
+                                px[u] = dev::load_pixel_slot<Src>(row, sx * static_cast<int>(sizeof(Src)), valid_lo, valid_hi);
+                            } else {
+                                const Src value = fetch(v, sx, sy);
+#pragma unroll
+                                for (int i = 0; i < SLOT; ++i) px[u].w[i] = 0u;
+                                __builtin_memcpy(px[u].w, &value, sizeof(Src));
+                            }
                         }
 #pragma unroll
-                        for (int i = 0; i < SLOT; ++i) tile[(r * stride + c) * SLOT + i] = px.w[i];
+                        for (int u = 0; u < STAGE_ROWS; ++u) {
+                            const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
+#pragma unroll
+                            for (int i = 0; i < SLOT; ++i) tile[(r * stride + c) * SLOT + i] = px[u].w[i];
+                        }
                     }
                 }
             }

@@ -203,6 +203,30 @@ FK_HD_CNST int floor_to_int(const float v) {
     return static_cast<float>(t) > v ? t - 1 : t;
 }
 FK_HD_CNST BilinearTaps bilinear_taps(const float src_x, const float src_y, const Size& srcSize) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if (!__builtin_is_constant_evaluated()) {
+        // The same values with fewer conversions: floor() is one instruction, and for |x| < 2^24 (any image) the float
+        // of x1 is floor(src_x) itself and the float of x1 + 1 is floor(src_x) + 1.
+        const float x1f = __builtin_floorf(src_x);
+#ifdef FK_INTERPOLATE_Y1_FROM_X
+        const float y1f = x1f;
+#else
+        const float y1f = __builtin_floorf(src_y);
+#endif
+        const int x1 = static_cast<int>(x1f), y1 = static_cast<int>(y1f);
+        const float x2f = x1f + 1.0f, y2f = y1f + 1.0f;
+        BilinearTaps t{};
+        t.x1 = x1;
+        t.y1 = y1;
+        t.x2r = x1 + 1 < srcSize.width - 1 ? x1 + 1 : srcSize.width - 1;
+        t.y2r = y1 + 1 < srcSize.height - 1 ? y1 + 1 : srcSize.height - 1;
+        t.wa = (x2f - src_x) * (y2f - src_y);
+        t.wb = (src_x - x1f) * (y2f - src_y);
+        t.wc = (x2f - src_x) * (src_y - y1f);
+        t.wd = (src_x - x1f) * (src_y - y1f);
+        return t;
+    }
+#endif
     const int x1 = floor_to_int(src_x);
 #ifdef FK_INTERPOLATE_Y1_FROM_X
     const int y1 = floor_to_int(src_x);
