@@ -113,10 +113,10 @@ __device__ __attribute__((always_inline)) inline void store_words(void* p, const
     }
 }
 
-// x / d with the host's r = RN(1 / d): the short form where every lane of the wave holds an x in [2^-60, 2^60], the
-// division instruction sequence elsewhere (the branch is wave-uniform).
+// x / d with the host's two-float reciprocal r + rl: the short form where every lane of the wave holds an x in
+// [2^-40, 2^40], the division instruction sequence elsewhere (the branch is wave-uniform).
 template <typename F>
-__device__ __attribute__((always_inline)) inline F prepared_divide(const F& x, const F& d, const float* r, const bool fast) {
+__device__ __attribute__((always_inline)) inline F prepared_divide(const F& x, const F& d, const float* r, const float* rl, const bool fast) {
     if (fast) {
         float lo = __builtin_fabsf(vectorAt(0, x)), hi = lo;
 #pragma unroll
@@ -132,8 +132,7 @@ __device__ __attribute__((always_inline)) inline F prepared_divide(const F& x, c
 #pragma unroll
             for (int c = 0; c < cn<F>; ++c) {
                 const float xc = vectorAt(c, x), dc = vectorAt(c, d), rc = r[c];
-                float qc = xc * rc;
-                qc = __builtin_fmaf(__builtin_fmaf(-dc, qc, xc), rc, qc);
+                float qc = __builtin_fmaf(xc, rc, xc * rl[c]);
                 qc = __builtin_fmaf(__builtin_fmaf(-dc, qc, xc), rc, qc);
                 q[c] = qc;
             }
@@ -151,7 +150,7 @@ __device__ __attribute__((always_inline)) inline auto compute_prepared(const V& 
     constexpr bool IS_DIV = IsFloatDiv<Op>::value;
     const auto step = [&] {
         if constexpr (IS_DIV && std::is_same_v<V, typename Op::InputType>) {
-            return prepared_divide(v, t.instance.params, tail.recip[I], (tail.fast >> I & 1u) != 0u);
+            return prepared_divide(v, t.instance.params, tail.recip[I], tail.recip_lo[I], (tail.fast >> I & 1u) != 0u);
         } else {
             return fk::detail::chain_step<Op>(Point(), v, t);
         }
@@ -566,12 +565,16 @@ __device__ __attribute__((always_inline)) inline PixelSlot<T> load_pixel_slot(co
     } else if constexpr (sizeof(T) == 3) {
         // one unaligned dword, [p, p + 4) for an aligned p and [p - 1, p + 3) otherwise: its one byte that is not the
         // pixel's lies in an aligned dword that also holds a byte of the pixel, so the load cannot fault and needs no
-        // branch (the loads of several rows are in flight together)
-        const char* const p = row + off;
-        const unsigned back = (static_cast<unsigned>(reinterpret_cast<size_t>(p)) & 3u) != 0u ? 1u : 0u;
-        unsigned int w;
-        __builtin_memcpy(&w, p - back, 4);
-        s.w[0] = w >> (8u * back);
+        // branch (the loads of several rows are in flight together).  `row` is the same for the whole wave: it stays
+        // in scalar registers and the lane adds a 32-bit offset, from row - 1 so that the offset is never negative.
+        struct __attribute__((packed)) UnalignedDword { unsigned int v; };
+        using GlobalBytes = const __attribute__((address_space(1))) char*;
+        using GlobalDword = const __attribute__((address_space(1))) UnalignedDword*;
+        GlobalBytes base = (GlobalBytes)(row - 1);
+        asm volatile("" : "+s"(base));
+        const unsigned aligned = ((static_cast<unsigned>(reinterpret_cast<size_t>(row)) + static_cast<unsigned>(off)) & 3u) == 0u ? 1u : 0u;
+        const unsigned int w = ((GlobalDword)(base + (static_cast<unsigned>(off) + aligned)))->v;
+        s.w[0] = aligned != 0u ? w : w >> 8u;
     } else {
         const unsigned mis = (static_cast<unsigned>(reinterpret_cast<size_t>(row)) + static_cast<unsigned>(off)) & 3u;
         const int first = off - static_cast<int>(mis); // aligned dword that holds the pixel's first byte

@@ -74,12 +74,12 @@ struct PlaneProgram {
 
 // ---- divisions by a divisor the host has seen ------------------------------------------------------------------------
 // A Div<float..> of a chain's tail divides every pixel by the same values.  IEEE division is eleven instructions on
-// this part; with r = RN(1 / d) from the host, q = x * r followed by two corrections q += fma(-d, q, x) * r is the
-// correctly rounded x / d as well (after the first correction q is RN(x / d + t) with |t| < 2^-23 ulp, hence a faithful
-// rounding; a correction of a faithful quotient by a correctly rounded reciprocal gives the correctly rounded quotient:
-// Markstein, "Computation of elementary functions on the IBM RISC System/6000 processor", 1990), as long as nothing on
-// the way leaves the normal range.  The host vouches for d (finite, 2^-60 <= |d| <= 2^60), the kernel tests x and takes
-// the division instruction sequence where a lane is outside (zeros, subnormals, infinities, huge values).
+// this part.  With the reciprocal as two floats from the host, r = RN(1 / d) and rl = RN(1 / d - r), four give the same
+// result: q = fma(x, r, x * rl) is x / d to a relative 2^-47 before its one rounding, hence a faithful quotient, and
+// the correction q + fma(-d, q, x) * r of a faithful quotient by a correctly rounded reciprocal is the correctly rounded
+// quotient (Markstein, "Computation of elementary functions on the IBM RISC System/6000 processor", 1990), as long as
+// nothing on the way leaves the normal range.  The host vouches for d (finite, 2^-40 <= |d| <= 2^40), the kernel tests x
+// and takes the division instruction sequence where a lane is outside (zeros, subnormals, infinities, huge values).
 template <typename Op>
 struct IsFloatDiv : std::false_type {};
 template <typename F>
@@ -87,13 +87,14 @@ struct IsFloatDiv<Div<F, F, F>> : std::bool_constant<std::is_same_v<VBase<F>, fl
 template <typename... Ops>
 constexpr int float_div_count = (0 + ... + (IsFloatDiv<Ops>::value ? 1 : 0));
 
-constexpr float PREPARED_DIV_LO = 8.67361738e-19f; // 2^-60
-constexpr float PREPARED_DIV_HI = 1.15292150e+18f; // 2^60
+constexpr float PREPARED_DIV_LO = 9.09494702e-13f; // 2^-40
+constexpr float PREPARED_DIV_HI = 1.09951163e+12f; // 2^40
 
 template <typename Ops, int NDIV>
 struct PreparedTail {
     Ops ops;
-    float recip[NDIV][4]; // per float division of the tail, in order: RN(1 / d) per channel
+    float recip[NDIV][4];    // per float division of the tail, in order: r = RN(1 / d) per channel
+    float recip_lo[NDIV][4]; // RN(1 / d - r)
     unsigned fast;        // bit i: every divisor of division i is in range, so its reciprocals are valid
 };
 
@@ -108,11 +109,17 @@ inline void prepare_divisions(Prepared& out, const OperationTuple<Op, Rest_...>&
     if constexpr (IS_DIV) {
         using F = typename Op::ParamsType;
         bool ok = true;
-        for (int c = 0; c < 4; ++c) out.recip[I][c] = 0.f;
+        for (int c = 0; c < 4; ++c) out.recip[I][c] = out.recip_lo[I][c] = 0.f;
         for (int c = 0; c < cn<F>; ++c) {
-            const volatile float d = vectorAt(c, t.instance.params); // volatile: a division at run time, correctly rounded
+            const volatile float d = vectorAt(c, t.instance.params); // volatile: divisions at run time, correctly rounded
             ok = ok && prepared_divisor_ok(d);
-            out.recip[I][c] = ok ? 1.0f / d : 0.f;
+            if (ok) {
+                const volatile float r = 1.0f / d;
+                // 1 / d in double is off by 2^-53 relative, far below the last bit of the float it is rounded to here
+                const volatile double rest = 1.0 / static_cast<double>(d) - static_cast<double>(r);
+                out.recip[I][c] = r;
+                out.recip_lo[I][c] = static_cast<float>(rest);
+            }
         }
         if (ok) out.fast |= 1u << I;
     }
@@ -289,7 +296,7 @@ struct ProgramOf<Read<FusedOperation<Head, ComputeOps...>>,
         if constexpr (std::is_same_v<Tail, Ops>) {
             return type{ ViewOf<Instantiable<Head>>::make(toIOp<Head>(iOp.params.instance)), fk::detail::tuple_tail(iOp.params) };
         } else {
-            type prog{ ViewOf<Instantiable<Head>>::make(toIOp<Head>(iOp.params.instance)), Tail{ fk::detail::tuple_tail(iOp.params), {}, 0u } };
+            type prog{ ViewOf<Instantiable<Head>>::make(toIOp<Head>(iOp.params.instance)), Tail{ fk::detail::tuple_tail(iOp.params), {}, {}, 0u } };
             detail::prepare_divisions<0>(prog.tail, prog.tail.ops);
             return prog;
         }
