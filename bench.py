@@ -48,10 +48,11 @@ class StreamTimer:
 SPINUP_S = 0.2
 
 
-def spin_up(launch, seconds=SPINUP_S):
+def spin_up(launch, seconds=None):
     """Untimed launches of the workload itself until the device has been busy for `seconds`: a process starts at idle
     clocks and the first milliseconds of launches run up to 20 % slower than the steady state that is measured."""
     import torch
+    seconds = SPINUP_S if seconds is None else seconds
     t0, i = time.perf_counter(), 0
     while time.perf_counter() - t0 < seconds:
         for _ in range(32):
@@ -243,10 +244,13 @@ def other_configs(fk, timer, steps, warmup, only=None):
 
 
 def main():
+    global SPINUP_S
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--spinup-s", type=float, default=SPINUP_S,
+                    help="seconds of untimed launches of each workload before its warm-up steps (shorter for traces)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-sweep", action="store_true", help="skip the depth sweep and the other configs")
     ap.add_argument("--only-config", default=None,
@@ -256,6 +260,7 @@ def main():
                     help="also run plain device copies of the same 99.5 MB image (torch copy kernel) before the timed "
                          "region, so that a counter run has a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
+    SPINUP_S = args.spinup_s
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (planes/row bands would shard with no "
                  "exchange); run with --gpus 1")

@@ -352,15 +352,22 @@ int main() {
             return static_cast<unsigned>(z ^ (z >> 31));
         };
         int mismatches = 0;
-        for (const float d : { 255.f, 6.f, 0.229f, 1e-30f, 3e38f, -7.f, 5e-39f, 1.f / 3.f }) {
+        // second pass per divisor: every operand within [2^-40, 2^40], where whole waves take the kernels' short division
+        // by the host's reciprocal instead of the division instruction sequence
+        for (const bool moderate : { false, true })
+        for (const float d : { 255.f, 6.f, 0.229f, 1e-30f, 3e38f, -7.f, 5e-39f, 1.f / 3.f, 1.99999988f, 1.00000012f, 57.375f, 9.5e-13f, 1.0e12f }) {
             for (uint i = 0; i < N; ++i) {
                 unsigned bits = next();
-                if (i % 4 == 1) bits &= 0x807fffffu;                        // subnormal operands
-                if (i % 4 == 2) bits = (bits & 0x80ffffffu) | 0x00800000u; // smallest normal operands
-                if (i % 64 == 3) bits = (i / 64 % 4 == 0) ? 0x7f800000u : (i / 64 % 4 == 1) ? 0xff800000u : (i / 64 % 4 == 2) ? 0x7fc00000u : 0x80000000u;
+                if (moderate) {
+                    bits = (bits & 0x807fffffu) | ((87u + next() % 80u) << 23);
+                } else {
+                    if (i % 4 == 1) bits &= 0x807fffffu;                        // subnormal operands
+                    if (i % 4 == 2) bits = (bits & 0x80ffffffu) | 0x00800000u; // smallest normal operands
+                    if (i % 64 == 3) bits = (i / 64 % 4 == 0) ? 0x7f800000u : (i / 64 % 4 == 1) ? 0xff800000u : (i / 64 % 4 == 2) ? 0x7fc00000u : 0x80000000u;
+                }
                 float v;
                 std::memcpy(&v, &bits, 4);
-                if (i % 4 == 3 && i < 4096) v = static_cast<float>(i / 4) * 1.40129846e-45f * d;
+                if (!moderate && i % 4 == 3 && i < 4096) v = static_cast<float>(i / 4) * 1.40129846e-45f * d;
                 in.at(i) = v;
             }
             in.upload(stream);
