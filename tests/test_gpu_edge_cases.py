@@ -130,6 +130,29 @@ def test_upscale_of_crops_with_odd_byte_offsets(fk, oracle):
         assert same_bits(out.cpu().numpy(), oracle.crop_resize_muls_bgr_tensor(src, rects, (150, 120), *args)), extra
 
 
+@pytest.mark.parametrize("case", ["behind", "shared", "mixed", "few_rows", "tall_boxes"])
+def test_resize_lds_layouts(fk, oracle, case):
+    """The resize kernel sizes its LDS from the planes' factors.  Packed outputs of 1 MB or more leave through LDS: behind
+    the source tile when both fit 24 KiB ("behind": up-scaling, small boxes), in the tile's place after a block barrier when
+    not ("shared": boxes above 12 KiB, down-scaling by 1.7); "mixed" has planes on both sides of that limit and one that is not staged at all in
+    one launch; "few_rows" are boxes of two or three source rows (a wave stages four rows at a time and repeats the last);
+    "tall_boxes" need more than one pass of four rows per wave."""
+    src = oracle.bytes(91, (720, 1280, 3))
+    rects, dst = {
+        "behind": ([(10, 20, 320, 200), (301, 7, 200, 320)], (768, 480)),
+        "shared": ([(0, 0, 1088, 626), (33, 11, 1090, 628)], (640, 368)),
+        "mixed": ([(5, 5, 160, 90), (0, 0, 1088, 626), (100, 50, 640, 368), (0, 0, 1280, 720), (600, 300, 17, 400)], (640, 368)),
+        "few_rows": ([(7, 300, 500, 3), (9, 100, 640, 2), (0, 0, 64, 1)], (1024, 512)),
+        "tall_boxes": ([(3, 1, 300, 700), (640, 0, 200, 720)], (512, 400)),
+    }[case]
+    for aspect in (B.IGNORE_AR, B.PRESERVE_AR):
+        args = (aspect, (0.5, 0.25, 0.125), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)
+        out = torch.full((len(rects), dst[1], dst[0], 3), float("nan"), device="cuda")
+        fk.crop_resize_muls_bgr_tensor(dev(src), rects, out, *args)
+        torch.cuda.synchronize()
+        assert same_bits(out.cpu().numpy(), oracle.crop_resize_muls_bgr_tensor(src, rects, dst, *args)), (case, aspect)
+
+
 def test_crop_at_the_last_row_and_column_of_the_buffer(fk, oracle):
     # the source window ends exactly at the end of the allocation: staging must not read past it
     src = oracle.bytes(81, (33, 47, 3))
