@@ -125,15 +125,22 @@ struct JobOf {
                 constexpr size_t out_elem = Out::IS_SPLIT ? sizeof(VBase<typename Out::Pixel>) : sizeof(typename Out::Pixel);
                 constexpr size_t out_chunk = dev::chunk_bytes(Job::K * static_cast<int>(out_elem));
                 int max_w = 0, max_h = 0;
+                bool flatten = Access::FLATTENS;
                 for (size_t i = 0; i < N; ++i) {
                     job.plane[i].prog = ProgramOf<PlaneIOp>::make(Planes::get(sender, i));
+                    if constexpr (Access::FLATTENS) {
+                        const auto& v = job.plane[i].prog.view;
+                        flatten = flatten && v.ox == 0 && v.oy == 0 && v.w == v.img_w && v.h > 1 &&
+                                  v.pitch == static_cast<uint>(v.w) * sizeof(Src) && out.pitch == static_cast<uint>(v.w) * out_elem &&
+                                  static_cast<size_t>(v.w) * v.h < (1u << 30);
+                    }
+                }
+                for (size_t i = 0; i < N; ++i) {
                     auto& v = job.plane[i].prog.view;
                     if constexpr (Access::FLATTENS) {
-                        if (N == 1 && v.ox == 0 && v.oy == 0 && v.w == v.img_w && v.h > 1 &&
-                            v.pitch == static_cast<uint>(v.w) * sizeof(Src) && out.pitch == static_cast<uint>(v.w) * out_elem &&
-                            static_cast<size_t>(v.w) * v.h < (1u << 30)) {
-                            // rows are contiguous on both sides: treat the image as one long row, so no block is cut
-                            // short at a row end
+                        if (flatten) {
+                            // rows are contiguous on both sides, in every plane: treat each image as one long row, so no
+                            // block is cut short at a row end
                             v.w = v.img_w = v.w * v.h;
                             v.h = v.img_h = 1;
                         }

@@ -475,6 +475,34 @@ public:
 
         using NewSeq = InstantiableOperationSequence<std::decay_t<decltype(newSender)>, std::decay_t<decltype(newReceiver)>>;
         using CopySeq = InstantiableOperationSequence<std::decay_t<decltype(copySender)>, std::decay_t<decltype(copyReceiver)>>;
+        if constexpr (BATCH > 1 && (std::is_same_v<WriteOp, TensorSplit<StoreT>> || std::is_same_v<WriteOp, TensorWrite<StoreT>>)) {
+            // In these two layouts a frame is one run of rows in the tensor and in the ring alike (its channel planes
+            // follow each other), so sequence 2 moves whole frames: the same copy as a batch of BATCH - 1 images read
+            // and written as they lie, which the executor runs with 16-byte accesses instead of one element at a time.
+            using E = std::remove_pointer_t<decltype(userWrite.params.data)>;
+            const auto& dst = userWrite.params;
+            const RawPtr<ND::_3D, E> ring = m_tempTensor.ptr();
+            const bool tight = dst.dims.plane_pitch == dst.dims.pitch * dst.dims.height && ring.dims.plane_pitch == ring.dims.pitch * ring.dims.height &&
+                               ring.dims.pitch == dst.dims.pitch && ring.dims.color_planes == dst.dims.color_planes;
+            if (tight) {
+                const uint rows = dst.dims.height * dst.dims.color_planes;
+                const size_t frame_bytes = static_cast<size_t>(dst.dims.pitch) * rows;
+                std::array<RawPtr<ND::_2D, E>, BATCH - 1> frames;
+                for (int i = 0; i < BATCH - 1; ++i) {
+                    const Point slot = circular_batch_internal::computeCircularThreadIdx<CTReadDirection_v<CT_ORDER>, BATCH>(Point(0, 0, FIRST_COPIED + i), m_nextUpdateIdx);
+                    frames[i] = RawPtr<ND::_2D, E>{ reinterpret_cast<E*>(reinterpret_cast<char*>(ring.data) + slot.z * frame_bytes),
+                                                   PtrDims<ND::_2D>(dst.dims.width, rows, dst.dims.pitch) };
+                }
+                const RawPtr<ND::_3D, E> copied{ reinterpret_cast<E*>(reinterpret_cast<char*>(dst.data) + FIRST_COPIED * frame_bytes),
+                                                 PtrDims<ND::_3D>(dst.dims.width, rows, BATCH - 1, 1, dst.dims.pitch) };
+                const auto framesSender = PerThreadRead<ND::_2D, E>::build(frames);
+                const auto framesReceiver = TensorWrite<E>::build(copied);
+                using FramesSeq = InstantiableOperationSequence<std::decay_t<decltype(framesSender)>, std::decay_t<decltype(framesReceiver)>>;
+                Executor<DivergentBatchTransformDPP<ParArch::GPU_AMD>>::executeOperations(stream, NewSeq{ newSender, newReceiver }, FramesSeq{ framesSender, framesReceiver });
+                m_nextUpdateIdx = (m_nextUpdateIdx + 1) % BATCH;
+                return;
+            }
+        }
         Executor<DivergentBatchTransformDPP<ParArch::GPU_AMD>>::executeOperations(stream, NewSeq{ newSender, newReceiver }, CopySeq{ copySender, copyReceiver });
         m_nextUpdateIdx = (m_nextUpdateIdx + 1) % BATCH;
     }
