@@ -257,6 +257,18 @@ __device__ __attribute__((always_inline)) inline void store_group(const SplitOut
         store_words<NB, STREAM && NB == chunk_bytes(NB)>(row + c * out.chan_stride + static_cast<size_t>(x0) * sizeof(B), w);
     }
 }
+// One or the other, chosen at run time (block-uniform).  The empty asm keeps the compiler from merging the two stores
+// into one plain store, which it does for stores that differ only in their cache hint.
+template <int K, typename Out, typename O>
+__device__ __attribute__((always_inline)) inline void store_group_either(const bool stream, const Out& out, int x0, int y, int z, const O* v) {
+    if (stream) {
+        asm volatile("" ::: "memory");
+        store_group<K, true>(out, x0, y, z, v);
+        asm volatile("" ::: "memory");
+    } else {
+        store_group<K>(out, x0, y, z, v);
+    }
+}
 } // namespace dev
 
 // Pixels per thread: the smallest power of two that makes the wider side a whole number of 16-byte transactions and
@@ -472,8 +484,7 @@ struct PointwiseJob {
                 }
             }
         } else if (active) {
-            if ((pl.flags & FLAG_STREAM_STORES) != 0u) dev::store_group<K, true>(job.out, x0, y, static_cast<int>(bz), o);
-            else dev::store_group<K>(job.out, x0, y, static_cast<int>(bz), o);
+            dev::store_group_either<K>((pl.flags & FLAG_STREAM_STORES) != 0u, job.out, x0, y, static_cast<int>(bz), o);
         }
     }
 
@@ -516,8 +527,7 @@ struct PointwiseJob {
             OutPixel o[K];
 #pragma unroll
             for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
-            if ((pl.flags & FLAG_STREAM_STORES) != 0u) dev::store_group<K, true>(job.out, x0, y, static_cast<int>(bz), o);
-            else dev::store_group<K>(job.out, x0, y, static_cast<int>(bz), o);
+            dev::store_group_either<K>((pl.flags & FLAG_STREAM_STORES) != 0u, job.out, x0, y, static_cast<int>(bz), o);
         } else {
             const int xe = x0 + K < v.w ? x0 + K : v.w;
             for (int x = x0; x < xe; ++x) {
@@ -841,28 +851,53 @@ struct ResizeJob {
 #pragma unroll
                 for (int j = 0; j < MINE; ++j) stage[tid * MINE + j] = mine[j];
                 dev::wave_sync();
-                const int wave_first = (tid >> 6) * (64 * MINE), lane = tid & 63;
-                char* const obase = reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
-                                    static_cast<size_t>(ty0) * job.out.pitch + static_cast<size_t>(tx0) * sizeof(OutPixel);
-                const int rows_here = v.h - ty0 < RESIZE_TILE_H ? v.h - ty0 : RESIZE_TILE_H;
+                // The wave's four rows start at a row address that is the same for all its lanes: it stays in scalar
+                // registers and a lane adds a 32-bit offset.  Instruction j of a lane covers piece j * 64 + lane of the
+                // wave's 4 * PIECES_PER_ROW: the end of row R0 for the lanes below THRESHOLD, the start of row R0 + 1
+                // for the others, both known at compile time, so no division and no 64-bit arithmetic per lane.
+                const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+                const int wave_first = wave * (64 * MINE);
+                using GlobalPiece = __attribute__((address_space(1))) dev::u32x4*;
+                using GlobalBytes = __attribute__((address_space(1))) char*;
+                GlobalBytes wbase = (GlobalBytes)(reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
+                                                  static_cast<size_t>(ty0 + 4 * wave) * job.out.pitch + static_cast<size_t>(tx0) * sizeof(OutPixel));
+                asm volatile("" : "+s"(wbase));
+                const int rows_here = (v.h - ty0 < RESIZE_TILE_H ? v.h - ty0 : RESIZE_TILE_H) - 4 * wave; // of this wave's four
                 const bool stream = (job.flags & FLAG_STREAM_STORES) != 0u;
+                const unsigned pitch = job.out.pitch;
+                // the two kinds of store in loops of their own: side by side in one loop body the compiler merges them
+                // into a plain store
+                const auto store_rows = [&](auto streaming) {
 #pragma unroll
-                for (int j = 0; j < MINE; ++j) {
-                    const int id = wave_first + j * 64 + lane;
-                    const int r = id / PIECES_PER_ROW, c = id - r * PIECES_PER_ROW;
-                    if (r < rows_here) {
-                        dev::u32x4* const g = reinterpret_cast<dev::u32x4*>(obase + static_cast<size_t>(r) * job.out.pitch) + c;
-                        if (stream) dev::store_piece<true>(g, stage[id]);
-                        else *g = stage[id];
+                    for (int j = 0; j < MINE; ++j) {
+                        constexpr int PPR = PIECES_PER_ROW;
+                        const int R0 = j * 64 / PPR;                   // row of the instruction's first piece
+                        const int THRESHOLD = (R0 + 1) * PPR - j * 64; // lanes from here on are in row R0 + 1
+                        const bool next_row = lane >= THRESHOLD;
+                        const unsigned row_off = next_row ? static_cast<unsigned>(R0 + 1) * pitch - static_cast<unsigned>(THRESHOLD) * 16u
+                                                          : static_cast<unsigned>(R0) * pitch + static_cast<unsigned>(j * 64 - R0 * PPR) * 16u;
+                        const int r = R0 + (next_row ? 1 : 0);
+                        if (r < rows_here) {
+                            const GlobalPiece g = (GlobalPiece)(wbase + (row_off + static_cast<unsigned>(lane) * 16u));
+                            const dev::u32x4 piece = stage[wave_first + j * 64 + lane];
+                            if constexpr (decltype(streaming)::value) __builtin_nontemporal_store(piece, g);
+                            else *g = piece;
+                        }
                     }
+                };
+                if (stream) {
+                    asm volatile("" ::: "memory"); // keep the streaming stores from being merged with the plain ones
+                    store_rows(std::true_type{});
+                    asm volatile("" ::: "memory");
+                } else {
+                    store_rows(std::false_type{});
                 }
                 return;
             }
         }
         if (y >= v.h) return;
         if (x_first + RESIZE_PX <= v.w && (job.flags & FLAG_VECTOR_IO) != 0u && (Out::IS_SPLIT || RESIZE_PX * sizeof(OutPixel) == 16)) {
-            if ((job.flags & FLAG_STREAM_STORES) != 0u) dev::store_group<RESIZE_PX, true>(job.out, x_first, y, static_cast<int>(bz), o);
-            else dev::store_group<RESIZE_PX>(job.out, x_first, y, static_cast<int>(bz), o);
+            dev::store_group_either<RESIZE_PX>((job.flags & FLAG_STREAM_STORES) != 0u, job.out, x_first, y, static_cast<int>(bz), o);
         } else {
 #pragma unroll
             for (int k = 0; k < RESIZE_PX; ++k) {
