@@ -701,7 +701,8 @@ struct ResizeJob {
                 Src a, b, c, d;
                 if constexpr (STAGED) {
                     // the tile holds columns sx_lo.. and rows sy_lo.., edge copies included: no clamping here
-                    const unsigned int* const p0 = tile + ((t.y1 - sy_lo) * stride + (t.x1 - sx_lo)) * SLOT;
+                    const unsigned int* const row0 = tile + ((t.y1 - sy_lo) * stride - sx_lo) * SLOT; // the same for the thread's four pixels
+                    const unsigned int* const p0 = row0 + t.x1 * SLOT;
                     const unsigned int* const p1 = p0 + stride * SLOT;
                     dev::PixelSlot<Src> sa, sb, sc, sd;
 #pragma unroll

@@ -214,16 +214,24 @@ FK_HD_CNST BilinearTaps bilinear_taps(const float src_x, const float src_y, cons
         const float y1f = __builtin_floorf(src_y);
 #endif
         const int x1 = static_cast<int>(x1f), y1 = static_cast<int>(y1f);
-        const float x2f = x1f + 1.0f, y2f = y1f + 1.0f;
+        // src_x - x1 is exact (x1 = floor(src_x) is at least half of src_x, or zero), so x2 - src_x, one rounding of
+        // 1 - (src_x - x1), is 1.0f minus that difference; the same for y
+        const float fx = src_x - x1f, fy = src_y - y1f;
+        const float gx = 1.0f - fx;
+#ifdef FK_INTERPOLATE_Y1_FROM_X
+        const float gy = (y1f + 1.0f) - src_y; // y1 is not the floor of src_y here: the difference above may be rounded
+#else
+        const float gy = 1.0f - fy;
+#endif
         BilinearTaps t{};
         t.x1 = x1;
         t.y1 = y1;
         t.x2r = x1 + 1 < srcSize.width - 1 ? x1 + 1 : srcSize.width - 1;
         t.y2r = y1 + 1 < srcSize.height - 1 ? y1 + 1 : srcSize.height - 1;
-        t.wa = (x2f - src_x) * (y2f - src_y);
-        t.wb = (src_x - x1f) * (y2f - src_y);
-        t.wc = (x2f - src_x) * (src_y - y1f);
-        t.wd = (src_x - x1f) * (src_y - y1f);
+        t.wa = gx * gy;
+        t.wb = fx * gy;
+        t.wc = gx * fy;
+        t.wd = fx * fy;
         return t;
     }
 #endif
