@@ -187,10 +187,22 @@ struct JobOf {
             job.active = sender.getActiveThreads();
             job.grid_x = job.plan(job.active);
             job.grid_y = ceil_div(job.active.y, 4u);
+            job.stream_rows = 0u;
+            if constexpr (decltype(job)::STREAMS_ROWS) {
+                const auto out = OutOf<Receiver>::make(receiver);
+                const size_t bytes = static_cast<size_t>(job.active.x) * job.active.y * job.active.z * sizeof(typename decltype(job)::Value);
+                const size_t piece = dev::chunk_bytes(static_cast<int>(sizeof(typename decltype(job)::Value)));
+                job.stream_rows = (bytes >= STREAM_STORE_MIN_BYTES && aligned_to(out.data, piece) && out.pitch % piece == 0u && out.z_stride % piece == 0u) ? 1u : 0u;
+                job.out_data = reinterpret_cast<char*>(out.data);
+                job.out_pitch = out.pitch;
+                job.out_z_stride = out.z_stride;
+            }
             job.packs_rows = 0u;
             if constexpr (decltype(job)::PACKS_ROWS) {
                 const auto out = OutOf<Receiver>::make(receiver);
                 job.packs_rows = (aligned_to(out.data, 4) && out.pitch % 4u == 0u && out.z_stride % 4u == 0u) ? 1u : 0u;
+                const size_t bytes = static_cast<size_t>(job.active.x) * job.active.y * job.active.z * sizeof(typename decltype(job)::Value);
+                job.stream_rows = (job.packs_rows != 0u && bytes >= STREAM_STORE_MIN_BYTES) ? 1u : 0u;
                 job.out_data = reinterpret_cast<char*>(out.data);
                 job.out_pitch = out.pitch;
                 job.out_z_stride = out.z_stride;

@@ -935,6 +935,15 @@ struct GenericJob {
     struct PacksRows<V, std::enable_if_t<V::supported>>
         : std::bool_constant<!V::type::IS_SPLIT && sizeof(typename V::type::Pixel) % 4 != 0 && std::is_same_v<typename V::type::Pixel, Value>> {};
     static constexpr bool PACKS_ROWS = PacksRows<OutView>::value;
+    // A packed receiver of whole-dword pixels (float3, float4, uchar4 ...): neighbouring lanes' stores make whole lines,
+    // so a large output is written with streaming stores, straight to the receiver's memory.
+    template <typename V, typename = void>
+    struct StreamsRows : std::false_type {};
+    template <typename V>
+    struct StreamsRows<V, std::enable_if_t<V::supported>>
+        : std::bool_constant<!V::type::IS_SPLIT && sizeof(typename V::type::Pixel) % 4 == 0 && std::is_same_v<typename V::type::Pixel, Value>> {};
+    static constexpr bool STREAMS_ROWS = StreamsRows<OutView>::value;
+    unsigned stream_rows; // decided by the host: large output, rows and planes at whole dwords (out_data etc. filled in)
     unsigned packs_rows; // the receiver's rows start at whole dwords (decided by the host, which then also fills in:)
     char* out_data;      // element (0, 0, 0) of the receiver, bytes between its rows and between its planes
     unsigned out_pitch;
@@ -970,7 +979,48 @@ struct GenericJob {
                 dev::pack_pixels<K>(value, words);
                 char* const run = job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch +
                                   static_cast<size_t>(x0) * S;
+                if (job.stream_rows != 0u) {
+                    asm volatile("" ::: "memory"); // keeps these stores apart from the plain ones (see store_group_either)
+                    if constexpr (S == 3) {
+                        typedef unsigned int u32x3 __attribute__((ext_vector_type(3)));
+                        typedef u32x3 __attribute__((aligned(4))) u32x3_dword_aligned;
+                        u32x3 v;
+                        v.x = words[0]; v.y = words[1]; v.z = words[2];
+                        __builtin_nontemporal_store(v, reinterpret_cast<u32x3_dword_aligned*>(run));
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < S; ++i) __builtin_nontemporal_store(words[i], reinterpret_cast<unsigned int*>(run) + i);
+                    }
+                    asm volatile("" ::: "memory");
+                    return;
+                }
                 __builtin_memcpy(__builtin_assume_aligned(run, 4), words, 4 * S);
+                return;
+            }
+        }
+        if constexpr (STREAMS_ROWS) {
+            if (job.stream_rows != 0u) {
+                constexpr int S = static_cast<int>(sizeof(Value));
+                char* const row = job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch;
+                asm volatile("" ::: "memory"); // keeps these stores apart from the plain ones below (see store_group_either)
+#pragma unroll
+                for (int k = 0; k < K; ++k) {
+                    if (x0 + STEP * k < w) {
+                        unsigned int words[S / 4];
+                        __builtin_memcpy(words, &value[k], S);
+                        char* const at = row + static_cast<size_t>(x0 + STEP * k) * S;
+                        if constexpr (S == 12) { // one three-dword store, as the plain form of a float3 is
+                            typedef unsigned int u32x3 __attribute__((ext_vector_type(3)));
+                            typedef u32x3 __attribute__((aligned(4))) u32x3_dword_aligned;
+                            u32x3 v;
+                            v.x = words[0]; v.y = words[1]; v.z = words[2];
+                            __builtin_nontemporal_store(v, reinterpret_cast<u32x3_dword_aligned*>(at));
+                        } else {
+                            dev::store_words<S, true>(at, words);
+                        }
+                    }
+                }
+                asm volatile("" ::: "memory");
                 return;
             }
         }
