@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused Transform path on one MI355X.
 
-Headline workload (BASELINE.json configs[1]): 3840x2160 float3, PerThreadRead -> 16 alternating Mul/Add ->
+Headline workload (the vertical-fusion configuration at depth 16): 3840x2160 float3, PerThreadRead -> 16 alternating Mul/Add ->
 PerThreadWrite in ONE launch.  One step = one fused launch over the whole image.  Inputs are resident in HBM before
 the timed region; three buffer sets (600 MB) are rotated so that the 256 MB Infinity Cache cannot hold a step's data.
 Prints ONE JSON line: Gpixel/s, the HBM roofline of the kernel (algorithmic bytes / measured duration vs 8 TB/s),
