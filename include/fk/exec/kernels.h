@@ -564,6 +564,17 @@ __device__ __attribute__((always_inline)) inline T slot_to_pixel(const PixelSlot
 // One pixel from memory at any byte alignment, as whole dwords.  `row` points at byte 0 of the window row, `off` is the
 // pixel's byte offset in it; [valid_lo, valid_hi) are the byte offsets of that row that belong to the parent image, so
 // dwords that would reach past them are assembled from single bytes.
+// The dword at byte `voff` from `row - 1`, for a `row` that is the same for the whole wave: the address stays in scalar
+// registers and the lane adds its 32-bit offset.
+__device__ __attribute__((always_inline)) inline unsigned int load_dword_from_row(const char* row, unsigned voff) {
+    struct __attribute__((packed)) UnalignedDword { unsigned int v; };
+    using GlobalBytes = const __attribute__((address_space(1))) char*;
+    using GlobalDword = const __attribute__((address_space(1))) UnalignedDword*;
+    GlobalBytes base = (GlobalBytes)(row - 1);
+    asm volatile("" : "+s"(base));
+    return ((GlobalDword)(base + voff))->v;
+}
+
 template <typename T>
 __device__ __attribute__((always_inline)) inline PixelSlot<T> load_pixel_slot(const char* row, int off, int valid_lo, int valid_hi) {
     constexpr int ND = slot_dwords<T>();
@@ -577,13 +588,8 @@ __device__ __attribute__((always_inline)) inline PixelSlot<T> load_pixel_slot(co
         // pixel's lies in an aligned dword that also holds a byte of the pixel, so the load cannot fault and needs no
         // branch (the loads of several rows are in flight together).  `row` is the same for the whole wave: it stays
         // in scalar registers and the lane adds a 32-bit offset, from row - 1 so that the offset is never negative.
-        struct __attribute__((packed)) UnalignedDword { unsigned int v; };
-        using GlobalBytes = const __attribute__((address_space(1))) char*;
-        using GlobalDword = const __attribute__((address_space(1))) UnalignedDword*;
-        GlobalBytes base = (GlobalBytes)(row - 1);
-        asm volatile("" : "+s"(base));
         const unsigned aligned = ((static_cast<unsigned>(reinterpret_cast<size_t>(row)) + static_cast<unsigned>(off)) & 3u) == 0u ? 1u : 0u;
-        const unsigned int w = ((GlobalDword)(base + (static_cast<unsigned>(off) + aligned)))->v;
+        const unsigned int w = load_dword_from_row(row, static_cast<unsigned>(off) + aligned);
         s.w[0] = aligned != 0u ? w : w >> 8u;
     } else {
         const unsigned mis = (static_cast<unsigned>(reinterpret_cast<size_t>(row)) + static_cast<unsigned>(off)) & 3u;
@@ -769,10 +775,10 @@ struct ResizeJob {
         if (resamples) {
             // source bounding box of the tile: taps are floor(c) and floor(c) + 1 for c in [lo, hi] * f; the column and
             // row past the source edge are staged as copies of the last one, which is what the clamp of the taps reads
-            sx_lo = fk::detail::floor_to_int((rx_lo - v.x1) * v.fx);
-            sy_lo = fk::detail::floor_to_int((ry_lo - v.y1) * v.fy);
-            const int cols = fk::detail::floor_to_int((rx_hi - v.x1) * v.fx) + 2 - sx_lo;
-            const int rows = fk::detail::floor_to_int((ry_hi - v.y1) * v.fy) + 2 - sy_lo;
+            sx_lo = static_cast<int>(__builtin_floorf((rx_lo - v.x1) * v.fx)); // the floor instruction; same value as floor_to_int
+            sy_lo = static_cast<int>(__builtin_floorf((ry_lo - v.y1) * v.fy));
+            const int cols = static_cast<int>(__builtin_floorf((rx_hi - v.x1) * v.fx)) + 2 - sx_lo;
+            const int rows = static_cast<int>(__builtin_floorf((ry_hi - v.y1) * v.fy)) + 2 - sy_lo;
             stride = cols | 1;
             const int tile_px = (rx_hi - rx_lo + 1) * (ry_hi - ry_lo + 1);
             // staging pays off while a source pixel is used about once or more; strong down-scaling reads taps directly
@@ -785,6 +791,34 @@ struct ResizeJob {
                 const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
                 constexpr int WAVES = BLOCK_THREADS / 64;
                 constexpr int STAGE_ROWS = SLOT == 1 ? 4 : 2;
+                bool rows_alike = false;
+                if constexpr (RAW_SOURCE && sizeof(Src) == 3) rows_alike = (s.pitch & 3u) == 0u;
+                if (rows_alike) {
+                    // three-byte pixels, rows a whole number of dwords apart: a column has the same alignment in every
+                    // row, so a lane's offset and the shift that takes the pixel out of its dword are found once per column
+                    if constexpr (RAW_SOURCE && sizeof(Src) == 3) {
+                        for (int c = lane; c < cols; c += 64) {
+                            const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
+                            const unsigned off = static_cast<unsigned>(sx) * 3u;
+                            const bool aligned = ((static_cast<unsigned>(reinterpret_cast<size_t>(window)) + off) & 3u) == 0u;
+                            const unsigned voff = off + (aligned ? 1u : 0u); // from one byte before the row
+                            for (int r0 = wave; r0 < rows; r0 += WAVES * STAGE_ROWS) {
+                                unsigned int w[STAGE_ROWS];
+#pragma unroll
+                                for (int u = 0; u < STAGE_ROWS; ++u) {
+                                    const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
+                                    const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
+                                    w[u] = dev::load_dword_from_row(window + static_cast<size_t>(sy) * s.pitch, voff);
+                                }
+#pragma unroll
+                                for (int u = 0; u < STAGE_ROWS; ++u) {
+                                    const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
+                                    tile[r * stride + c] = aligned ? w[u] : w[u] >> 8u;
+                                }
+                            }
+                        }
+                    }
+                } else
                 for (int c = lane; c < cols; c += 64) {
                     const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
                     for (int r0 = wave; r0 < rows; r0 += WAVES * STAGE_ROWS) {
