@@ -902,7 +902,7 @@ struct ResizeJob {
                 const unsigned pitch = job.out.pitch;
                 // the two kinds of store in loops of their own: side by side in one loop body the compiler merges them
                 // into a plain store
-                const auto store_rows = [&](auto streaming) {
+                const auto store_rows = [&](auto streaming, auto all_rows) { // all_rows: the wave's four rows lie in the plane
 #pragma unroll
                     for (int j = 0; j < MINE; ++j) {
                         constexpr int PPR = PIECES_PER_ROW;
@@ -912,7 +912,7 @@ struct ResizeJob {
                         const unsigned row_off = next_row ? static_cast<unsigned>(R0 + 1) * pitch - static_cast<unsigned>(THRESHOLD) * 16u
                                                           : static_cast<unsigned>(R0) * pitch + static_cast<unsigned>(j * 64 - R0 * PPR) * 16u;
                         const int r = R0 + (next_row ? 1 : 0);
-                        if (r < rows_here) {
+                        if (decltype(all_rows)::value || r < rows_here) {
                             const GlobalPiece g = (GlobalPiece)(wbase + (row_off + static_cast<unsigned>(lane) * 16u));
                             const dev::u32x4 piece = stage[wave_first + j * 64 + lane];
                             if constexpr (decltype(streaming)::value) __builtin_nontemporal_store(piece, g);
@@ -922,10 +922,11 @@ struct ResizeJob {
                 };
                 if (stream) {
                     asm volatile("" ::: "memory"); // keep the streaming stores from being merged with the plain ones
-                    store_rows(std::true_type{});
+                    if (rows_here >= 4) store_rows(std::true_type{}, std::true_type{});
+                    else store_rows(std::true_type{}, std::false_type{});
                     asm volatile("" ::: "memory");
                 } else {
-                    store_rows(std::false_type{});
+                    store_rows(std::false_type{}, std::false_type{});
                 }
                 return;
             }
