@@ -133,6 +133,15 @@ def other_configs(fk, timer, steps, warmup, only=None):
         record("C1_scaled_5x1024x768_to_1920x1080", ms, 5 * 1920 * 1080, 5 * 1024 * 768 * 3 + 5 * 1920 * 1080 * 12)
         del out1s, calls
 
+    # the same with 16:9 crops: no bars, every output pixel is resampled
+    if want("C1_nobars_5x1024x576_to_1920x1080"):
+        rects_n = [(64 * i, 48 * i, 1024, 576) for i in range(5)]
+        out1n = [torch.empty((5, 1080, 1920, 3), device="cuda") for _ in range(3)]
+        calls = [fk.crop_resize_muls_bgr_tensor(img4k, rects_n, o, *a1, defer=True) for o in out1n]
+        ms = time_launches(timer, lambda i: calls[i % 3](), steps, warmup)
+        record("C1_nobars_5x1024x576_to_1920x1080", ms, 5 * 1920 * 1080, 5 * 1024 * 576 * 3 + 5 * 1920 * 1080 * 12)
+        del out1n, calls
+
     # C3: 50 crops of 50 images -> 224x224x3x50 planar
     if want("C3_batch50_224x224_split"):
         imgs = [rnd_u8(1080, 1920, 3) for _ in range(50)]

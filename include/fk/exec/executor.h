@@ -7,6 +7,7 @@
 #ifndef FK_EXEC_EXECUTOR_H
 #define FK_EXEC_EXECUTOR_H
 
+#include <cstdlib>
 #include <cstring>
 #include <tuple>
 #include <memory>
@@ -52,6 +53,15 @@ inline unsigned ceil_div(unsigned a, unsigned b) { return (a + b - 1u) / b; }
 #endif
 constexpr size_t STREAM_STORE_MIN_BYTES = static_cast<size_t>(FK_STREAM_STORE_MIN_MIB) << 20;
 inline bool aligned_to(const void* p, size_t a) { return reinterpret_cast<size_t>(p) % a == 0; }
+// FK_RESIZE_WAVE_ROWS=4|8|16 fixes the resize kernel's tile height (64 x 4 * rows) instead of the choice made per launch:
+// for measurements.
+inline unsigned resize_wave_rows_override() {
+    static const unsigned rows = [] {
+        const char* env = std::getenv("FK_RESIZE_WAVE_ROWS");
+        return env != nullptr ? static_cast<unsigned>(std::strtoul(env, nullptr, 10)) : 0u;
+    }();
+    return rows;
+}
 
 // ---- job construction ----------------------------------------------------------------------------------------
 namespace detail {
@@ -112,16 +122,15 @@ struct JobOf {
                 }
                 job.out = out;
                 job.grid_x = ceil_div(static_cast<unsigned>(max_w), RESIZE_TILE_W);
-                job.grid_y = ceil_div(static_cast<unsigned>(max_h), RESIZE_TILE_H);
-                // vector stores need 16-byte aligned rows in every plane (tiles start at multiples of 64 pixels)
-                constexpr size_t out_elem = Out::IS_SPLIT ? sizeof(VBase<typename Out::Pixel>) : sizeof(typename Out::Pixel);
-                bool vec = aligned_to(out.data, 16) && out.pitch % 16 == 0 && out.z_stride % 16 == 0 && (RESIZE_TILE_W * out_elem) % 16 == 0;
-                if constexpr (Out::IS_SPLIT) vec = vec && out.chan_stride % 16 == 0;
-                const bool stream = static_cast<size_t>(max_w) * max_h * N * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
-                job.flags = (vec ? FLAG_VECTOR_IO : 0u) | (vec && stream ? FLAG_STREAM_STORES : 0u);
-                // small outputs gain nothing from leaving through LDS, and the LDS they would ask for lowers occupancy
-                if (vec && static_cast<size_t>(max_w) * max_h * N * sizeof(typename Out::Pixel) >= (1u << 20)) job.flags |= FLAG_STAGE_OUT;
-                job.plan_lds(); // sets FLAG_SOURCE_TILE when some plane's tiles are worth staging
+                // streaming stores for large outputs whose rows, planes and channel planes start at whole dwords
+                bool dwords = aligned_to(out.data, 4) && out.pitch % 4 == 0 && out.z_stride % 4 == 0;
+                // (the kernel addresses a wave's rows, and their channel planes, with 32-bit offsets from its first row)
+                if constexpr (Out::IS_SPLIT) dwords = dwords && out.chan_stride % 4 == 0 && out.chan_stride * 4 + static_cast<size_t>(out.pitch) * 64 < (1u << 30);
+                dwords = dwords && static_cast<size_t>(out.pitch) * 64 < (1u << 30);
+                const bool large = static_cast<size_t>(max_w) * max_h * N * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
+                job.flags = dwords && large ? FLAG_STREAM_STORES : 0u;
+                // tile height, grid rows and LDS layout; sets FLAG_SOURCE_TILE when some plane's tiles are worth staging
+                job.grid_y = job.plan(max_h, resize_wave_rows_override());
                 return job;
             } else {
                 using Job = PointwiseJob<Prog, N, Out>;

@@ -37,6 +37,48 @@ namespace dev {
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
+// Streaming stores: `nt` keeps the written lines from displacing what the kernel still reads, `sc1` (device scope)
+// sends them on to memory at once instead of holding them in the writer's L2; together they measured 3-4 % above `nt`
+// alone on a write-only stream (6.06 against 5.79 TB/s in this kernel family's tile pattern).  Only for accesses where
+// a wave writes whole cache lines (consecutive lanes, consecutive pieces).  The pair of bits is reachable through the
+// buffer form of the store: a descriptor of the memory from an address on that is the same for the whole wave (it
+// stays in scalar registers), a per-lane and a per-wave byte offset.
+typedef unsigned int u32x3 __attribute__((ext_vector_type(3)));
+constexpr int STREAM_POLICY = 0x12;            // nt | sc1
+constexpr int WAVE_BUFFER_BYTES = 0x7fffffff;  // offsets are checked against this range; stores beyond it are dropped
+__device__ __attribute__((always_inline)) inline __amdgpu_buffer_rsrc_t wave_buffer(void* wave_uniform_base) {
+    return __builtin_amdgcn_make_buffer_rsrc(wave_uniform_base, 0, WAVE_BUFFER_BYTES, 0x00020000);
+}
+template <int ND, typename Words> // ND dwords (a three-element vector is as large as a four-element one)
+__device__ __attribute__((always_inline)) inline void stream_store_at(const __amdgpu_buffer_rsrc_t buffer, const unsigned lane_offset,
+                                                                    const unsigned wave_offset, const Words v) {
+    static_assert(ND >= 1 && ND <= 4, "one to four dwords");
+    if constexpr (ND == 1) __builtin_amdgcn_raw_buffer_store_b32(v, buffer, lane_offset, wave_offset, STREAM_POLICY);
+    else if constexpr (ND == 2) __builtin_amdgcn_raw_buffer_store_b64(v, buffer, lane_offset, wave_offset, STREAM_POLICY);
+    else if constexpr (ND == 3) __builtin_amdgcn_raw_buffer_store_b96(v, buffer, lane_offset, wave_offset, STREAM_POLICY);
+    else __builtin_amdgcn_raw_buffer_store_b128(v, buffer, lane_offset, wave_offset, STREAM_POLICY);
+}
+// the same address in every lane, for the compiler to see
+__device__ __attribute__((always_inline)) inline char* wave_uniform(char* p) {
+    const size_t a = reinterpret_cast<size_t>(p);
+    const unsigned lo = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(a)));
+    const unsigned hi = static_cast<unsigned>(__builtin_amdgcn_readfirstlane(static_cast<int>(a >> 32)));
+    return reinterpret_cast<char*>(static_cast<size_t>(hi) << 32 | lo);
+}
+// a pixel of 1-4 whole dwords as a register vector
+template <typename O>
+struct WordsOf {
+    static constexpr int ND = static_cast<int>(sizeof(O)) / 4;
+    typedef unsigned int vec_t __attribute__((ext_vector_type(ND == 1 ? 2 : ND))); // (a one-element vector type does not exist)
+    using type = std::conditional_t<ND == 1, unsigned int, vec_t>;
+    __device__ __attribute__((always_inline)) static inline type of(const O& v) {
+        type w;
+        __builtin_memcpy(&w, &v, sizeof(O));
+        return w;
+    }
+};
+
+
 __device__ __attribute__((always_inline)) inline int thread_in_block() { return static_cast<int>(__builtin_amdgcn_workitem_id_x()); }
 __device__ __attribute__((always_inline)) inline void block_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -385,7 +427,7 @@ struct SourceAccess<YuvView<PF>> {
 };
 
 // ---- pointwise ---------------------------------------------------------------------------------------------------
-enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_STAGE_OUT = 8u };
+enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u };
 
 template <typename Prog, size_t N, typename Out>
 struct PointwiseJob {
@@ -473,9 +515,11 @@ struct PointwiseJob {
                 static_cast<size_t>(y) * job.out.pitch + static_cast<size_t>(bx0) * sizeof(OutPixel)) + wave * (64 * MINE);
             const int pieces = span * static_cast<int>(sizeof(OutPixel)) / 16 - wave * (64 * MINE);
             if ((pl.flags & FLAG_STREAM_STORES) != 0u) {
+                // the wave's span starts at the same address for all its lanes
+                const __amdgpu_buffer_rsrc_t span_buffer = dev::wave_buffer(dev::wave_uniform(reinterpret_cast<char*>(g)));
 #pragma unroll
                 for (int j = 0; j < MINE; ++j) {
-                    if (FULL || j * 64 + lane < pieces) dev::store_piece<true>(g + j * 64 + lane, stage[j * 64 + lane]);
+                    if (FULL || j * 64 + lane < pieces) dev::stream_store_at<4>(span_buffer, static_cast<unsigned>(j * 64 + lane) * 16u, 0u, stage[j * 64 + lane]);
                 }
             } else {
 #pragma unroll
@@ -539,12 +583,14 @@ struct PointwiseJob {
 };
 
 // ---- resize ------------------------------------------------------------------------------------------------------
-// A block owns a 64x16 output tile of one plane; a thread computes four consecutive pixels of one row, so everything
-// that depends only on the row (or only on the column) is computed once and shared.
+// A block owns an output tile of one plane, 64 columns by 4 * wave_rows rows: each of its four waves wave_rows rows of it
+// (4, 8 or 16, chosen per launch), each lane one column of those.
 constexpr int RESIZE_TILE_W = 64;
-constexpr int RESIZE_TILE_H = 16;
-constexpr int RESIZE_PX = 4;                // pixels per thread, along x
-constexpr int RESIZE_LDS_DWORDS = 6144;     // source tile capacity (24 KiB)
+constexpr int RESIZE_GROUP_ROWS = 4;      // rows that a wave finishes, and writes, at a time
+constexpr int RESIZE_MAX_WAVE_ROWS = 16;
+constexpr int RESIZE_LDS_DWORDS = 6144;   // source tile capacity (24 KiB)
+constexpr size_t RESIZE_MIN_BLOCKS = 4096; // a taller tile is chosen only while the grid keeps this many blocks
+static_assert(RESIZE_TILE_W == 64, "a lane per column");
 
 namespace dev {
 // LDS slot of one source pixel: whole dwords, so a tap is one aligned LDS read whatever the pixel's byte size
@@ -626,118 +672,195 @@ struct ResizeJob {
     using Src = typename View::Source; // the pixel that is interpolated: the source view's pixel after Pre
     using Pixel = typename View::Pixel;
     using OutPixel = typename Out::Pixel;
-    // packed pixels read as they are: taps and tile slots come straight from memory as dwords
+    // packed pixels read as they are: taps and staged pixels come straight from memory as dwords
     static constexpr bool RAW_SOURCE = std::is_same_v<SrcView, PlainView<Src>> && std::is_same_v<Pre, NoTail>;
-    static constexpr int SLOT = dev::slot_dwords<Src>();
-    static constexpr int OUT_ROW_BYTES = RESIZE_TILE_W * static_cast<int>(sizeof(OutPixel));
-    // packed outputs whose four pixels per thread are not one 16-byte piece go out through LDS as whole 16-byte pieces
-    static constexpr bool STAGE_OUT = !Out::IS_SPLIT && (RESIZE_PX * sizeof(OutPixel)) % 16 == 0 && RESIZE_PX * sizeof(OutPixel) > 16;
-    static constexpr int OUT_STAGE_BYTES = STAGE_OUT ? RESIZE_TILE_H * OUT_ROW_BYTES : 0;
+    // What is interpolated: the channels of a source pixel as floats, which is what the blend makes of them anyway
+    // (a channel times a float weight).  The tile holds them in that form, so a source pixel is converted once, when it
+    // is staged, however many output pixels tap it.  Channels of doubles or 64-bit integers stay as they are and are
+    // promoted by the blend itself.
+    using Tap = std::conditional_t<(sizeof(VBase<Src>) <= 4), Pixel, Src>;
+    static_assert(sizeof(Tap) % 4 == 0, "a tap is whole dwords");
+    static constexpr int SLOT = static_cast<int>(sizeof(Tap)) / 4; // dwords of a source pixel in the tile
     static constexpr bool READ_IN_PLACE = N > 1;
     Prog plane[N];
     Out out;
     unsigned grid_x, grid_y;
-    // FLAG_VECTOR_IO: output rows start 16-byte aligned; FLAG_STREAM_STORES: large output; FLAG_SOURCE_TILE: some plane's
-    // tiles are worth staging in LDS; FLAG_STAGE_OUT: packed output leaves through LDS.  The last two decide how much
-    // LDS the launch asks for (a divergent launch shares one LDS size between all its jobs).
+    // FLAG_STREAM_STORES: large output whose rows start at whole dwords; FLAG_SOURCE_TILE: some plane's tiles are worth
+    // staging in LDS, which decides how much LDS the launch asks for (a divergent launch shares one LDS size between all
+    // its jobs).
     unsigned flags;
+    // Rows of the tile that each of the block's four waves computes (4, 8 or 16: the tile is 64 x 4 * wave_rows).
+    // What a wave does once (the tile's source box, its lanes' columns) is shared by more rows in a taller tile; a
+    // launch of few tiles keeps them small so that the grid still fills the device.
+    unsigned wave_rows;
     // The launch asks for as much LDS as the planes' own factors need, not for the capacity: a block's LDS decides how
-    // many blocks a CU holds.  tile_dwords is the room for a source tile (a tile that needs more reads its taps
-    // directly); the packed output is staged behind it when both fit the capacity (out_stage_offset, in bytes), else in
-    // the same place (0), which costs a block barrier between the last tap and the first staged pixel.
+    // many blocks a CU holds.  tile_dwords is the room for a source tile (a tile that needs more reads its taps directly).
     unsigned tile_dwords;
-    unsigned out_stage_offset;
-    size_t lds_bytes() const {
-        size_t n = 0;
-        if ((flags & FLAG_SOURCE_TILE) != 0u) n = static_cast<size_t>(tile_dwords) * 4;
-        if (STAGE_OUT && (flags & FLAG_STAGE_OUT) != 0u && out_stage_offset + static_cast<size_t>(OUT_STAGE_BYTES) > n) n = out_stage_offset + OUT_STAGE_BYTES;
-        return n == 0 ? 0 : n + 16;
-    }
+    size_t lds_bytes() const { return (flags & FLAG_SOURCE_TILE) != 0u ? static_cast<size_t>(tile_dwords) * 4 + 16 : 0; }
+    int tile_h() const { return (BLOCK_THREADS / 64) * static_cast<int>(wave_rows); }
     // dwords a tile of a plane with these factors takes when staged, 0 when it is not worth staging (same rule as the
     // kernel applies per tile)
-    static unsigned staged_tile_dwords(float fx, float fy) {
-        const int cols = static_cast<int>((RESIZE_TILE_W - 1) * fx) + 3, rows = static_cast<int>((RESIZE_TILE_H - 1) * fy) + 3;
-        const bool worth = rows * (cols | 1) * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * RESIZE_TILE_W * RESIZE_TILE_H + 256;
+    static unsigned staged_tile_dwords(float fx, float fy, int tile_h) {
+        // strong down-scaling is never staged; this also keeps the factors of a plane whose resized image has no
+        // extent at all (infinite: such a plane is all background) out of the integer arithmetic below
+        if (!(fx >= 0.f && fx <= 8.f && fy >= 0.f && fy <= 8.f)) return 0u;
+        const int cols = static_cast<int>((RESIZE_TILE_W - 1) * fx) + 3, rows = static_cast<int>((tile_h - 1) * fy) + 3;
+        const bool worth = rows * (cols | 1) * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * RESIZE_TILE_W * tile_h + 256;
         return worth ? static_cast<unsigned>(rows * (cols | 1) * SLOT) : 0u;
     }
-    // fills in the LDS layout from the planes' factors; FLAG_STAGE_OUT has been decided
-    void plan_lds() {
+    // Chooses the tile height and the LDS size from the planes' factors; grid_x has been decided, max_h is the tallest
+    // plane.  Returns the number of tile rows (grid_y).
+    unsigned plan(int max_h, unsigned forced_wave_rows) {
+        // the tallest tile that still leaves two rounds of blocks for every CU's eight block slots, and whose source
+        // boxes fit the LDS wherever those of the smallest tile do
+        const auto blocks = [&](unsigned wr) { return static_cast<size_t>(N) * grid_x * ((static_cast<unsigned>(max_h) + 4u * wr - 1u) / (4u * wr)); };
+        const auto staged_planes = [&](unsigned wr) {
+            unsigned n = 0;
+            for (size_t i = 0; i < N; ++i) n += staged_tile_dwords(plane[i].view.fx, plane[i].view.fy, 4 * static_cast<int>(wr)) != 0u ? 1u : 0u;
+            return n;
+        };
+        wave_rows = RESIZE_GROUP_ROWS;
+        for (unsigned wr = RESIZE_MAX_WAVE_ROWS; wr > RESIZE_GROUP_ROWS; wr /= 2) {
+            if (blocks(wr) >= RESIZE_MIN_BLOCKS && staged_planes(wr) == staged_planes(RESIZE_GROUP_ROWS)) {
+                wave_rows = wr;
+                break;
+            }
+        }
+        if (forced_wave_rows == 4u || forced_wave_rows == 8u || forced_wave_rows == 16u) wave_rows = forced_wave_rows;
         tile_dwords = 0;
         for (size_t i = 0; i < N; ++i) {
-            const unsigned need = staged_tile_dwords(plane[i].view.fx, plane[i].view.fy);
+            const unsigned need = staged_tile_dwords(plane[i].view.fx, plane[i].view.fy, tile_h());
             tile_dwords = need > tile_dwords ? need : tile_dwords;
         }
-        tile_dwords = (tile_dwords + 3u) & ~3u; // what follows the tile starts at a whole 16 bytes
         if (tile_dwords != 0u) flags |= FLAG_SOURCE_TILE;
-        const bool behind = STAGE_OUT && (flags & FLAG_STAGE_OUT) != 0u && tile_dwords * 4u + OUT_STAGE_BYTES <= RESIZE_LDS_DWORDS * 4u;
-        out_stage_offset = behind ? tile_dwords * 4u : 0u;
+        return (static_cast<unsigned>(max_h) + static_cast<unsigned>(tile_h()) - 1u) / static_cast<unsigned>(tile_h());
     }
 
     // source pixel (x, y) of the resampled window, after the operations fused before the resize
     __device__ __attribute__((always_inline)) static inline Src fetch(const View& v, int x, int y) {
         return dev::apply_tail(v.pre, Access::load_one(v.src, x, y));
     }
+    __device__ __attribute__((always_inline)) static inline Tap to_tap(const Src& p) {
+        if constexpr (std::is_same_v<Tap, Src>) return p;
+        else return fk::detail::cast_channels<Tap>(p);
+    }
+    __device__ __attribute__((always_inline)) static inline Tap load_tap(const unsigned int* p) {
+        unsigned int w[SLOT];
+#pragma unroll
+        for (int k = 0; k < SLOT; ++k) w[k] = p[k];
+        Tap t;
+        __builtin_memcpy(&t, w, sizeof(Tap));
+        return t;
+    }
+    __device__ __attribute__((always_inline)) static inline void store_tap(unsigned int* p, const Tap& t) {
+        unsigned int w[SLOT];
+        __builtin_memcpy(w, &t, sizeof(Tap));
+#pragma unroll
+        for (int k = 0; k < SLOT; ++k) p[k] = w[k];
+    }
+    __device__ __attribute__((always_inline)) static inline float lane_float(const float value, const int lane) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, value), lane));
+    }
 
-    // Four consecutive pixels of row y, taps from the staged tile (STAGED) or straight from memory.
-    template <bool STAGED, bool INTERIOR>
-    __device__ __attribute__((always_inline)) static inline void pixels(const Prog& prog, const unsigned int* tile, const char* window,
-                                                                       int sx_lo, int sy_lo, int stride, int x_first, int y, OutPixel* o) {
+    // The rows of a wave (rows wy0 .. wy0 + wave_rows - 1 of the plane), one column per lane (column x), four rows at a
+    // time.  What depends on the column alone is computed once for all the rows.  What depends on the row alone is the
+    // same for the whole wave: lane i (i < wave_rows) computes it for row i and it is read from there.
+    // `put(g, k, pixel)` takes the finished pixel of row g + k (g the group's first row, k = 0..3 known at compile time).
+    template <bool STAGED, bool INTERIOR, typename Put>
+    __device__ __attribute__((always_inline)) static inline void sweep(const Prog& prog, const unsigned int* tile, const char* window, const int sx_lo,
+                                                                      const int sy_lo, const int stride, const int x, const int wy0, const int lane,
+                                                                      const int wave_rows, const Put& put) {
         const View& v = prog.view;
         const SrcView& s = v.src;
-        const int ry = y + v.off_y;
-        bool row_inside = INTERIOR || y < v.h;
-        if constexpr (View::HAS_ROI && !INTERIOR) row_inside = row_inside && ry >= v.y1 && ry <= v.y2;
-        const float src_y = (ry - v.y1) * v.fy;
         // a short tail is taken into registers once, ahead of the pixels (read in place it is fetched where it is used,
         // once per pixel and with the wait in the middle of the arithmetic)
         using Tail = std::decay_t<decltype(prog.tail)>;
         const std::conditional_t<(sizeof(Tail) <= 128), Tail, const Tail&> tail = prog.tail;
-        // the float of (rx - x1) for the thread's first pixel; the next ones are that plus 1, 2, 3 (exact: far below 2^24)
-        const float rel_x0 = static_cast<float>(x_first + v.off_x - v.x1);
-#pragma unroll
-        for (int k = 0; k < RESIZE_PX; ++k) {
-            const int x = x_first + k;
-            const int rx = x + v.off_x;
-            bool inside = INTERIOR || (row_inside && x < v.w);
-            if constexpr (View::HAS_ROI && !INTERIOR) inside = inside && rx >= v.x1 && rx <= v.x2;
-            Pixel value = v.background;
-            if (inside) {
-                const float src_x = (rel_x0 + static_cast<float>(k)) * v.fx;
-                const fk::detail::BilinearTaps t = fk::detail::bilinear_taps(src_x, src_y, Size(s.w, s.h));
-                Src a, b, c, d;
-                if constexpr (STAGED) {
-                    // the tile holds columns sx_lo.. and rows sy_lo.., edge copies included: no clamping here
-                    const unsigned int* const row0 = tile + ((t.y1 - sy_lo) * stride - sx_lo) * SLOT; // the same for the thread's four pixels
-                    const unsigned int* const p0 = row0 + t.x1 * SLOT;
-                    const unsigned int* const p1 = p0 + stride * SLOT;
-                    dev::PixelSlot<Src> sa, sb, sc, sd;
-#pragma unroll
-                    for (int i = 0; i < SLOT; ++i) {
-                        sa.w[i] = p0[i];
-                        sb.w[i] = p0[SLOT + i];
-                        sc.w[i] = p1[i];
-                        sd.w[i] = p1[SLOT + i];
-                    }
-                    a = dev::slot_to_pixel<Src>(sa);
-                    b = dev::slot_to_pixel<Src>(sb);
-                    c = dev::slot_to_pixel<Src>(sc);
-                    d = dev::slot_to_pixel<Src>(sd);
-                } else if constexpr (RAW_SOURCE) {
-                    const Src* const r0 = reinterpret_cast<const Src*>(window + static_cast<size_t>(t.y1) * s.pitch);
-                    const Src* const r1 = reinterpret_cast<const Src*>(window + static_cast<size_t>(t.y2r) * s.pitch);
-                    a = fk::detail::read_element(r0 + t.x1);
-                    b = fk::detail::read_element(r0 + t.x2r);
-                    c = fk::detail::read_element(r1 + t.x1);
-                    d = fk::detail::read_element(r1 + t.x2r);
-                } else {
-                    a = fetch(v, t.x1, t.y1);
-                    b = fetch(v, t.x2r, t.y1);
-                    c = fetch(v, t.x1, t.y2r);
-                    d = fetch(v, t.x2r, t.y2r);
-                }
-                value = fk::detail::bilinear_blend(a, b, c, d, t);
+
+        // ---- this lane's column ----
+        const int rx = x + v.off_x;
+        bool col_in = INTERIOR || x < v.w;
+        if constexpr (View::HAS_ROI && !INTERIOR) col_in = col_in && rx >= v.x1 && rx <= v.x2;
+        const float src_x = static_cast<float>(rx - v.x1) * v.fx;
+        // floor() in float: for |x| < 2^24 the float of x1 is floor(src_x) itself, src_x - x1 is exact, and x2 - src_x,
+        // one rounding of 1 - (src_x - x1), is 1.0f minus that difference (fk::detail::bilinear_taps)
+        const float x1f = __builtin_floorf(src_x);
+        const float wx1 = src_x - x1f, wx0 = 1.0f - wx1;
+        const int x1 = col_in ? static_cast<int>(x1f) : sx_lo; // a column beside the image reads (and discards) a valid tap
+
+        // ---- row (lane & 15) of the wave, for the lanes that are asked for it ----
+        const int yi = wy0 + (lane & (RESIZE_MAX_WAVE_ROWS - 1));
+        const int ry = yi + v.off_y;
+        bool row_in = INTERIOR || yi < v.h;
+        if constexpr (View::HAS_ROI && !INTERIOR) row_in = row_in && ry >= v.y1 && ry <= v.y2;
+        const float src_y = static_cast<float>(ry - v.y1) * v.fy;
+        const float y1f = __builtin_floorf(src_y);
+        const float wy1 = src_y - y1f, wy0f = 1.0f - wy1;
+        const int y1 = row_in ? static_cast<int>(y1f) : sy_lo;
+        unsigned rows_in = 0xFFFFu;
+        if constexpr (!INTERIOR) rows_in = static_cast<unsigned>(__builtin_amdgcn_ballot_w64(row_in)) & 0xFFFFu;
+
+        const auto emit = [&](const int g, const auto k, const Tap& a, const Tap& b, const Tap& c, const Tap& d) {
+            const int i = g + decltype(k)::value;
+            const float gy = lane_float(wy0f, i), fy = lane_float(wy1, i);
+            fk::detail::BilinearTaps t{};
+            t.wa = wx0 * gy;
+            t.wb = wx1 * gy;
+            t.wc = wx0 * fy;
+            t.wd = wx1 * fy;
+            Pixel value = fk::detail::bilinear_blend(a, b, c, d, t);
+            if constexpr (!INTERIOR) {
+                if (!(col_in && (rows_in >> i & 1u) != 0u)) value = v.background;
             }
-            o[k] = dev::apply_tail(tail, value);
+            put(g, k, dev::apply_tail(tail, value));
+        };
+        const auto each_of_group = [](const auto& body) {
+            body(std::integral_constant<int, 0>{});
+            body(std::integral_constant<int, 1>{});
+            body(std::integral_constant<int, 2>{});
+            body(std::integral_constant<int, 3>{});
+        };
+        static_assert(RESIZE_GROUP_ROWS == 4, "the group is written out above");
+
+        if constexpr (STAGED) {
+            // the tile holds columns sx_lo.. and rows sy_lo.., edge copies included: no clamping here
+            const unsigned int* const column = tile + (x1 - sx_lo) * SLOT;
+            const int row_dwords = stride * SLOT;
+            const int tile_row = y1 - sy_lo;
+            for (int g = 0; g < wave_rows; g += RESIZE_GROUP_ROWS) {
+                each_of_group([&](const auto k) {
+                    const unsigned int* const p = column + __builtin_amdgcn_readlane(tile_row, g + decltype(k)::value) * row_dwords;
+                    emit(g, k, load_tap(p), load_tap(p + SLOT), load_tap(p + row_dwords), load_tap(p + row_dwords + SLOT));
+                });
+            }
+        } else {
+            // taps straight from memory, those of a group's four rows requested before the first is used
+            const int x2 = x1 + 1 < s.w - 1 ? x1 + 1 : s.w - 1;
+            const int y2 = y1 + 1 < s.h - 1 ? y1 + 1 : s.h - 1;
+            for (int g = 0; g < wave_rows; g += RESIZE_GROUP_ROWS) {
+                Src a[RESIZE_GROUP_ROWS], b[RESIZE_GROUP_ROWS], c[RESIZE_GROUP_ROWS], d[RESIZE_GROUP_ROWS];
+#pragma unroll
+                for (int k = 0; k < RESIZE_GROUP_ROWS; ++k) {
+                    const int ya = __builtin_amdgcn_readlane(y1, g + k), yb = __builtin_amdgcn_readlane(y2, g + k);
+                    if constexpr (RAW_SOURCE) {
+                        const Src* const r0 = reinterpret_cast<const Src*>(window + static_cast<size_t>(ya) * s.pitch);
+                        const Src* const r1 = reinterpret_cast<const Src*>(window + static_cast<size_t>(yb) * s.pitch);
+                        a[k] = fk::detail::read_element(r0 + x1);
+                        b[k] = fk::detail::read_element(r0 + x2);
+                        c[k] = fk::detail::read_element(r1 + x1);
+                        d[k] = fk::detail::read_element(r1 + x2);
+                    } else {
+                        a[k] = fetch(v, x1, ya);
+                        b[k] = fetch(v, x2, ya);
+                        c[k] = fetch(v, x1, yb);
+                        d[k] = fetch(v, x2, yb);
+                    }
+                }
+                each_of_group([&](const auto k) {
+                    constexpr int K = decltype(k)::value;
+                    emit(g, k, to_tap(a[K]), to_tap(b[K]), to_tap(c[K]), to_tap(d[K]));
+                });
+            }
         }
     }
 
@@ -745,16 +868,16 @@ struct ResizeJob {
         const Prog& prog = job.plane[N == 1 ? 0u : bz];
         const View& v = prog.view;
         const SrcView& s = v.src;
+        const int wave_rows = static_cast<int>(job.wave_rows);
+        const int tile_h = (BLOCK_THREADS / 64) * wave_rows;
         const int tx0 = static_cast<int>(bx) * RESIZE_TILE_W;
-        const int ty0 = static_cast<int>(by) * RESIZE_TILE_H;
+        const int ty0 = static_cast<int>(by) * tile_h;
         if (tx0 >= v.w || ty0 >= v.h) return; // block outside this plane's own extent
         const int tid = dev::thread_in_block();
-        const int x_first = tx0 + (tid & (RESIZE_TILE_W / RESIZE_PX - 1)) * RESIZE_PX;
-        const int y = ty0 + tid / (RESIZE_TILE_W / RESIZE_PX);
 
         // part of the tile that resamples the source, in resize coordinates (after the outer crop offset)
         int rx_lo = tx0 + v.off_x, rx_hi = (tx0 + RESIZE_TILE_W < v.w ? tx0 + RESIZE_TILE_W : v.w) - 1 + v.off_x;
-        int ry_lo = ty0 + v.off_y, ry_hi = (ty0 + RESIZE_TILE_H < v.h ? ty0 + RESIZE_TILE_H : v.h) - 1 + v.off_y;
+        int ry_lo = ty0 + v.off_y, ry_hi = (ty0 + tile_h < v.h ? ty0 + tile_h : v.h) - 1 + v.off_y;
         if constexpr (View::HAS_ROI) {
             rx_lo = rx_lo > v.x1 ? rx_lo : v.x1;
             rx_hi = rx_hi < v.x2 ? rx_hi : v.x2;
@@ -766,7 +889,7 @@ struct ResizeJob {
         unsigned int* const tile = reinterpret_cast<unsigned int*>(lds_raw);
         bool staged = false;
         int sx_lo = 0, sy_lo = 0;
-        int stride = 0; // slots per tile row
+        int stride = 0; // source pixels per tile row
         // window pixel (0, 0) and the byte range of a window row that belongs to the parent image (raw sources only)
         const char* const window = reinterpret_cast<const char*>(s.data) + static_cast<size_t>(s.oy) * s.pitch +
                                    static_cast<size_t>(s.ox) * sizeof(Src);
@@ -790,7 +913,7 @@ struct ResizeJob {
                 // compiler moves the load to the store and waits there.
                 const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
                 constexpr int WAVES = BLOCK_THREADS / 64;
-                constexpr int STAGE_ROWS = SLOT == 1 ? 4 : 2;
+                constexpr int STAGE_ROWS = sizeof(Src) <= 4 ? 4 : 2;
                 bool rows_alike = false;
                 if constexpr (RAW_SOURCE && sizeof(Src) == 3) rows_alike = (s.pitch & 3u) == 0u;
                 if (rows_alike) {
@@ -813,7 +936,9 @@ struct ResizeJob {
 #pragma unroll
                                 for (int u = 0; u < STAGE_ROWS; ++u) {
                                     const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
-                                    tile[r * stride + c] = aligned ? w[u] : w[u] >> 8u;
+                                    dev::PixelSlot<Src> px;
+                                    px.w[0] = aligned ? w[u] : w[u] >> 8u;
+                                    store_tap(tile + (r * stride + c) * SLOT, to_tap(dev::slot_to_pixel<Src>(px)));
                                 }
                             }
                         }
@@ -822,26 +947,22 @@ struct ResizeJob {
                 for (int c = lane; c < cols; c += 64) {
                     const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
                     for (int r0 = wave; r0 < rows; r0 += WAVES * STAGE_ROWS) {
-                        dev::PixelSlot<Src> px[STAGE_ROWS];
+                        Src px[STAGE_ROWS];
 #pragma unroll
                         for (int u = 0; u < STAGE_ROWS; ++u) {
                             const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
                             const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
                             if constexpr (RAW_SOURCE) {
                                 const char* const row = window + static_cast<size_t>(sy) * s.pitch;
-                                px[u] = dev::load_pixel_slot<Src>(row, sx * static_cast<int>(sizeof(Src)), valid_lo, valid_hi);
+                                px[u] = dev::slot_to_pixel<Src>(dev::load_pixel_slot<Src>(row, sx * static_cast<int>(sizeof(Src)), valid_lo, valid_hi));
                             } else {
-                                const Src value = fetch(v, sx, sy);
-#pragma unroll
-                                for (int i = 0; i < SLOT; ++i) px[u].w[i] = 0u;
-                                __builtin_memcpy(px[u].w, &value, sizeof(Src));
+                                px[u] = fetch(v, sx, sy);
                             }
                         }
 #pragma unroll
                         for (int u = 0; u < STAGE_ROWS; ++u) {
                             const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
-#pragma unroll
-                            for (int i = 0; i < SLOT; ++i) tile[(r * stride + c) * SLOT + i] = px[u].w[i];
+                            store_tap(tile + (r * stride + c) * SLOT, to_tap(px[u]));
                         }
                     }
                 }
@@ -849,97 +970,79 @@ struct ResizeJob {
         }
         dev::block_sync();
 
-        // ---- this thread's four pixels; the tap source is decided once for the block ----
-        OutPixel o[RESIZE_PX];
+        // ---- compute: a wave owns wave_rows rows of the tile, a lane one column of them ----
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+        const int x = tx0 + lane;
+        const int wy0 = ty0 + wave_rows * wave;
+        if (wy0 >= v.h) return; // the plane ends above this wave's rows (no barrier follows)
+        const bool whole_width = tx0 + RESIZE_TILE_W <= v.w; // block-uniform
         // interior tiles (whole tile inside the plane and inside the region that holds the image) need no per-pixel tests
-        bool interior = tx0 + RESIZE_TILE_W <= v.w && ty0 + RESIZE_TILE_H <= v.h;
+        bool interior = whole_width && ty0 + tile_h <= v.h;
         if constexpr (View::HAS_ROI) {
             interior = interior && tx0 + v.off_x >= v.x1 && tx0 + RESIZE_TILE_W - 1 + v.off_x <= v.x2 && ty0 + v.off_y >= v.y1 &&
-                       ty0 + RESIZE_TILE_H - 1 + v.off_y <= v.y2;
+                       ty0 + tile_h - 1 + v.off_y <= v.y2;
         }
-        if (!resamples) {
-            // a tile that lies wholly beside the image (the bars of a preserved aspect ratio): one value for all of it
-            const OutPixel bar = dev::apply_tail(prog.tail, v.background);
-#pragma unroll
-            for (int k = 0; k < RESIZE_PX; ++k) o[k] = bar;
-        } else if (staged) {
-            if (interior) pixels<true, true>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
-            else pixels<true, false>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
-        } else {
-            if (interior) pixels<false, true>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
-            else pixels<false, false>(prog, tile, window, sx_lo, sy_lo, stride, x_first, y, o);
-        }
-
-        // ---- write ----
-        const bool whole_width = tx0 + RESIZE_TILE_W <= v.w; // block-uniform
-        if constexpr (STAGE_OUT) {
-            if (whole_width && (job.flags & FLAG_STAGE_OUT) != 0u) {
-                constexpr int PIECES_PER_ROW = OUT_ROW_BYTES / 16;
-                constexpr int MINE = RESIZE_PX * static_cast<int>(sizeof(OutPixel)) / 16;
-                dev::u32x4* const stage = reinterpret_cast<dev::u32x4*>(lds_raw + job.out_stage_offset);
-                // the buffer held the source tile: every thread is done with it
-                if (job.out_stage_offset == 0u && (job.flags & FLAG_SOURCE_TILE) != 0u) dev::block_sync();
-                // A wave's 64 threads own four whole rows of the tile (64 * MINE pieces), so a wave moves its rows
-                // through its own part of the buffer and never waits for the other waves of the block.
-                dev::u32x4 mine[MINE];
-                __builtin_memcpy(mine, o, sizeof(mine));
-#pragma unroll
-                for (int j = 0; j < MINE; ++j) stage[tid * MINE + j] = mine[j];
-                dev::wave_sync();
-                // The wave's four rows start at a row address that is the same for all its lanes: it stays in scalar
-                // registers and a lane adds a 32-bit offset.  Instruction j of a lane covers piece j * 64 + lane of the
-                // wave's 4 * PIECES_PER_ROW: the end of row R0 for the lanes below THRESHOLD, the start of row R0 + 1
-                // for the others, both known at compile time, so no division and no 64-bit arithmetic per lane.
-                const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-                const int wave_first = wave * (64 * MINE);
-                using GlobalPiece = __attribute__((address_space(1))) dev::u32x4*;
-                using GlobalBytes = __attribute__((address_space(1))) char*;
-                GlobalBytes wbase = (GlobalBytes)(reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
-                                                  static_cast<size_t>(ty0 + 4 * wave) * job.out.pitch + static_cast<size_t>(tx0) * sizeof(OutPixel));
-                asm volatile("" : "+s"(wbase));
-                const int rows_here = (v.h - ty0 < RESIZE_TILE_H ? v.h - ty0 : RESIZE_TILE_H) - 4 * wave; // of this wave's four
-                const bool stream = (job.flags & FLAG_STREAM_STORES) != 0u;
-                const unsigned pitch = job.out.pitch;
-                // the two kinds of store in loops of their own: side by side in one loop body the compiler merges them
-                // into a plain store
-                const auto store_rows = [&](auto streaming, auto all_rows) { // all_rows: the wave's four rows lie in the plane
-#pragma unroll
-                    for (int j = 0; j < MINE; ++j) {
-                        constexpr int PPR = PIECES_PER_ROW;
-                        const int R0 = j * 64 / PPR;                   // row of the instruction's first piece
-                        const int THRESHOLD = (R0 + 1) * PPR - j * 64; // lanes from here on are in row R0 + 1
-                        const bool next_row = lane >= THRESHOLD;
-                        const unsigned row_off = next_row ? static_cast<unsigned>(R0 + 1) * pitch - static_cast<unsigned>(THRESHOLD) * 16u
-                                                          : static_cast<unsigned>(R0) * pitch + static_cast<unsigned>(j * 64 - R0 * PPR) * 16u;
-                        const int r = R0 + (next_row ? 1 : 0);
-                        if (decltype(all_rows)::value || r < rows_here) {
-                            const GlobalPiece g = (GlobalPiece)(wbase + (row_off + static_cast<unsigned>(lane) * 16u));
-                            const dev::u32x4 piece = stage[wave_first + j * 64 + lane];
-                            if constexpr (decltype(streaming)::value) __builtin_nontemporal_store(piece, g);
-                            else *g = piece;
+        // the whole computation exists once per kind of put
+        const auto compute = [&](const auto& put) {
+            if (!resamples) {
+                // a tile that lies wholly beside the image (the bars of a preserved aspect ratio): one value for all of it
+                const OutPixel bar = dev::apply_tail(prog.tail, v.background);
+                for (int g = 0; g < wave_rows; g += RESIZE_GROUP_ROWS) {
+                    put(g, std::integral_constant<int, 0>{}, bar);
+                    put(g, std::integral_constant<int, 1>{}, bar);
+                    put(g, std::integral_constant<int, 2>{}, bar);
+                    put(g, std::integral_constant<int, 3>{}, bar);
+                }
+            } else if (staged) {
+                if (interior) sweep<true, true>(prog, tile, window, sx_lo, sy_lo, stride, x, wy0, lane, wave_rows, put);
+                else sweep<true, false>(prog, tile, window, sx_lo, sy_lo, stride, x, wy0, lane, wave_rows, put);
+            } else {
+                if (interior) sweep<false, true>(prog, tile, window, sx_lo, sy_lo, stride, x, wy0, lane, wave_rows, put);
+                else sweep<false, false>(prog, tile, window, sx_lo, sy_lo, stride, x, wy0, lane, wave_rows, put);
+            }
+        };
+        // One pixel per lane straight from registers: a wave's store covers 64 neighbouring pixels of a row (768
+        // consecutive bytes of 12-byte pixels: as fast as 16-byte pieces, measured, and nothing passes through LDS).
+        const Out out = job.out;
+        const bool column_here = x < v.w;
+        const int rows_here = v.h - wy0; // rows from the wave's first to the plane's last (may exceed the wave's own)
+        constexpr bool CAN_STREAM = Out::IS_SPLIT ? sizeof(VBase<OutPixel>) == 4 : (sizeof(OutPixel) % 4 == 0 && sizeof(OutPixel) <= 16);
+        if constexpr (CAN_STREAM) {
+            if ((job.flags & FLAG_STREAM_STORES) != 0u) {
+                // the address of the wave's first row is the same in all its lanes: a descriptor from there on, the row as
+                // the wave's offset (in a scalar register) and the column as the lane's
+                const __amdgpu_buffer_rsrc_t rows = dev::wave_buffer(dev::wave_uniform(
+                    reinterpret_cast<char*>(out.data) + static_cast<size_t>(bz) * out.z_stride + static_cast<size_t>(wy0) * out.pitch));
+                const unsigned pitch = out.pitch;
+                if constexpr (Out::IS_SPLIT) {
+                    const unsigned at = static_cast<unsigned>(x) * 4u;
+                    const unsigned chan_stride = static_cast<unsigned>(out.chan_stride); // the host has checked that all offsets fit
+                    compute([&](const int g, const auto k, const OutPixel& o) {
+                        const int i = g + decltype(k)::value;
+                        if (column_here && i < rows_here) {
+                            const unsigned row = static_cast<unsigned>(i) * pitch;
+                            dev::stream_store_at<1>(rows, at, row, __builtin_bit_cast(unsigned int, o.x));
+                            dev::stream_store_at<1>(rows, at, row + chan_stride, __builtin_bit_cast(unsigned int, o.y));
+                            if constexpr (cn<OutPixel> >= 3) dev::stream_store_at<1>(rows, at, row + 2u * chan_stride, __builtin_bit_cast(unsigned int, o.z));
+                            if constexpr (cn<OutPixel> == 4) dev::stream_store_at<1>(rows, at, row + 3u * chan_stride, __builtin_bit_cast(unsigned int, o.w));
                         }
-                    }
-                };
-                if (stream) {
-                    asm volatile("" ::: "memory"); // keep the streaming stores from being merged with the plain ones
-                    if (rows_here >= 4) store_rows(std::true_type{}, std::true_type{});
-                    else store_rows(std::true_type{}, std::false_type{});
-                    asm volatile("" ::: "memory");
+                    });
                 } else {
-                    store_rows(std::false_type{}, std::false_type{});
+                    const unsigned at = static_cast<unsigned>(x) * static_cast<unsigned>(sizeof(OutPixel));
+                    compute([&](const int g, const auto k, const OutPixel& o) {
+                        const int i = g + decltype(k)::value;
+                        if (column_here && i < rows_here) {
+                            dev::stream_store_at<dev::WordsOf<OutPixel>::ND>(rows, at, static_cast<unsigned>(i) * pitch, dev::WordsOf<OutPixel>::of(o));
+                        }
+                    });
                 }
                 return;
             }
         }
-        if (y >= v.h) return;
-        if (x_first + RESIZE_PX <= v.w && (job.flags & FLAG_VECTOR_IO) != 0u && (Out::IS_SPLIT || RESIZE_PX * sizeof(OutPixel) == 16)) {
-            dev::store_group_either<RESIZE_PX>((job.flags & FLAG_STREAM_STORES) != 0u, job.out, x_first, y, static_cast<int>(bz), o);
-        } else {
-#pragma unroll
-            for (int k = 0; k < RESIZE_PX; ++k) {
-                if (x_first + k < v.w) dev::store_one(job.out, x_first + k, y, static_cast<int>(bz), o[k]);
-            }
-        }
+        compute([&](const int g, const auto k, const OutPixel& o) {
+            const int i = g + decltype(k)::value;
+            if (column_here && i < rows_here) dev::store_one(out, x, wy0 + i, static_cast<int>(bz), o);
+        });
     }
 };
 
@@ -1015,18 +1118,18 @@ struct GenericJob {
                 char* const run = job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch +
                                   static_cast<size_t>(x0) * S;
                 if (job.stream_rows != 0u) {
-                    asm volatile("" ::: "memory"); // keeps these stores apart from the plain ones (see store_group_either)
+                    // the row is the same for the whole wave (a wave is one row of the block)
+                    const __amdgpu_buffer_rsrc_t row_buffer = dev::wave_buffer(dev::wave_uniform(
+                        job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch));
+                    const unsigned at = static_cast<unsigned>(x0) * S;
                     if constexpr (S == 3) {
-                        typedef unsigned int u32x3 __attribute__((ext_vector_type(3)));
-                        typedef u32x3 __attribute__((aligned(4))) u32x3_dword_aligned;
-                        u32x3 v;
+                        dev::u32x3 v;
                         v.x = words[0]; v.y = words[1]; v.z = words[2];
-                        __builtin_nontemporal_store(v, reinterpret_cast<u32x3_dword_aligned*>(run));
+                        dev::stream_store_at<3>(row_buffer, at, 0u, v);
                     } else {
 #pragma unroll
-                        for (int i = 0; i < S; ++i) __builtin_nontemporal_store(words[i], reinterpret_cast<unsigned int*>(run) + i);
+                        for (int i = 0; i < S; ++i) dev::stream_store_at<1>(row_buffer, at + 4u * i, 0u, words[i]);
                     }
-                    asm volatile("" ::: "memory");
                     return;
                 }
                 __builtin_memcpy(__builtin_assume_aligned(run, 4), words, 4 * S);
@@ -1036,26 +1139,28 @@ struct GenericJob {
         if constexpr (STREAMS_ROWS) {
             if (job.stream_rows != 0u) {
                 constexpr int S = static_cast<int>(sizeof(Value));
-                char* const row = job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch;
-                asm volatile("" ::: "memory"); // keeps these stores apart from the plain ones below (see store_group_either)
+                // the row is the same for the whole wave (a wave is one row of the block)
+                const __amdgpu_buffer_rsrc_t row_buffer = dev::wave_buffer(dev::wave_uniform(
+                    job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch));
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
                     if (x0 + STEP * k < w) {
-                        unsigned int words[S / 4];
-                        __builtin_memcpy(words, &value[k], S);
-                        char* const at = row + static_cast<size_t>(x0 + STEP * k) * S;
-                        if constexpr (S == 12) { // one three-dword store, as the plain form of a float3 is
-                            typedef unsigned int u32x3 __attribute__((ext_vector_type(3)));
-                            typedef u32x3 __attribute__((aligned(4))) u32x3_dword_aligned;
-                            u32x3 v;
-                            v.x = words[0]; v.y = words[1]; v.z = words[2];
-                            __builtin_nontemporal_store(v, reinterpret_cast<u32x3_dword_aligned*>(at));
+                        const unsigned at = static_cast<unsigned>(x0 + STEP * k) * S;
+                        if constexpr (S <= 16) {
+                            dev::stream_store_at<S / 4>(row_buffer, at, 0u, dev::WordsOf<Value>::of(value[k]));
                         } else {
-                            dev::store_words<S, true>(at, words);
+                            unsigned int words[S / 4];
+                            __builtin_memcpy(words, &value[k], S);
+#pragma unroll
+                            for (int i = 0; i < S / 16; ++i) {
+                                dev::u32x4 piece;
+                                piece.x = words[4 * i]; piece.y = words[4 * i + 1]; piece.z = words[4 * i + 2]; piece.w = words[4 * i + 3];
+                                dev::stream_store_at<4>(row_buffer, at + 16u * i, 0u, piece);
+                            }
+                            static_assert(S <= 16 || S % 16 == 0, "larger pixels are whole 16-byte pieces");
                         }
                     }
                 }
-                asm volatile("" ::: "memory");
                 return;
             }
         }

@@ -85,6 +85,24 @@ def test_c5_divergent_full_size(fk, oracle):
     assert np.array_equal(c, np.minimum(window, 255).astype(np.uint8))
 
 
+README_ARGS = ((0, 0, 0), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)
+
+
+@pytest.mark.parametrize("crop", [(1024, 768), (1024, 576)], ids=["4x3_with_bars", "16x9_no_bars"])
+@pytest.mark.parametrize("aspect", [B.PRESERVE_AR, B.IGNORE_AR, B.PRESERVE_AR_RN_EVEN, B.PRESERVE_AR_LEFT])
+def test_readme_pipeline_bandwidth_sized(fk, oracle, crop, aspect):
+    """The README chain at the shapes its roofline figures are quoted on: five crops of a 4K frame -> 1920x1080 each.
+    The 4:3 crops leave bars of background under PRESERVE_AR; the 16:9 crops resample every output pixel."""
+    src = oracle.bytes(11, (2160, 3840, 3))
+    cw, ch = crop
+    rects = [(64 * i, 48 * i, cw, ch) for i in range(5)]
+    want = oracle.crop_resize_muls_bgr_tensor(src, rects, (1920, 1080), aspect, *README_ARGS)
+    out = torch.full((5, 1080, 1920, 3), float("nan"), device="cuda")
+    fk.crop_resize_muls_bgr_tensor(dev(src), rects, out, aspect, *README_ARGS)
+    torch.cuda.synchronize()
+    assert same_bits(out.cpu().numpy(), want)
+
+
 def test_c1_readme_matches_reference_vectors_where_defined(fk, oracle):
     """The committed vectors come from the reference's CPU backend, whose host branch takes the bilinear row from x;
     on every element where that equals the row from y the GPU must reproduce the reference's own bits."""
