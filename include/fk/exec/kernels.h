@@ -589,7 +589,9 @@ constexpr int RESIZE_TILE_W = 64;
 constexpr int RESIZE_GROUP_ROWS = 4;      // rows that a wave finishes, and writes, at a time
 constexpr int RESIZE_MAX_WAVE_ROWS = 16;
 constexpr int RESIZE_LDS_DWORDS = 6144;   // source tile capacity (24 KiB)
-constexpr size_t RESIZE_MIN_BLOCKS = 4096; // a taller tile is chosen only while the grid keeps this many blocks
+// A taller tile is chosen only while the grid keeps this many blocks (measured: 50 planes of 224 x 224 are faster as 1400
+// tiles of 64 x 32 than as 2800 of 64 x 16, five planes of 1920 x 1080 slower as 2550 tiles of 64 x 64 than as 5100 of 64 x 32).
+constexpr size_t RESIZE_MIN_BLOCKS_16 = 4096, RESIZE_MIN_BLOCKS_8 = 1024;
 static_assert(RESIZE_TILE_W == 64, "a lane per column");
 
 namespace dev {
@@ -711,8 +713,8 @@ struct ResizeJob {
     // Chooses the tile height and the LDS size from the planes' factors; grid_x has been decided, max_h is the tallest
     // plane.  Returns the number of tile rows (grid_y).
     unsigned plan(int max_h, unsigned forced_wave_rows) {
-        // the tallest tile that still leaves two rounds of blocks for every CU's eight block slots, and whose source
-        // boxes fit the LDS wherever those of the smallest tile do
+        // the tallest tile that still leaves the grid enough blocks, and whose source boxes fit the LDS wherever those of
+        // the smallest tile do
         const auto blocks = [&](unsigned wr) { return static_cast<size_t>(N) * grid_x * ((static_cast<unsigned>(max_h) + 4u * wr - 1u) / (4u * wr)); };
         const auto staged_planes = [&](unsigned wr) {
             unsigned n = 0;
@@ -720,12 +722,8 @@ struct ResizeJob {
             return n;
         };
         wave_rows = RESIZE_GROUP_ROWS;
-        for (unsigned wr = RESIZE_MAX_WAVE_ROWS; wr > RESIZE_GROUP_ROWS; wr /= 2) {
-            if (blocks(wr) >= RESIZE_MIN_BLOCKS && staged_planes(wr) == staged_planes(RESIZE_GROUP_ROWS)) {
-                wave_rows = wr;
-                break;
-            }
-        }
+        if (blocks(16) >= RESIZE_MIN_BLOCKS_16 && staged_planes(16) == staged_planes(RESIZE_GROUP_ROWS)) wave_rows = 16;
+        else if (blocks(8) >= RESIZE_MIN_BLOCKS_8 && staged_planes(8) == staged_planes(RESIZE_GROUP_ROWS)) wave_rows = 8;
         if (forced_wave_rows == 4u || forced_wave_rows == 8u || forced_wave_rows == 16u) wave_rows = forced_wave_rows;
         tile_dwords = 0;
         for (size_t i = 0; i < N; ++i) {
@@ -837,6 +835,42 @@ struct ResizeJob {
             // taps straight from memory, those of a group's four rows requested before the first is used
             const int x2 = x1 + 1 < s.w - 1 ? x1 + 1 : s.w - 1;
             const int y2 = y1 + 1 < s.h - 1 ? y1 + 1 : s.h - 1;
+            if constexpr (RAW_SOURCE && sizeof(Src) == 3) {
+                if ((s.pitch & 3u) == 0u) {
+                    // Three-byte pixels, rows a whole number of dwords apart: a column has the same alignment in every
+                    // row, so the offset of the dword that holds the pixel (from one byte before the row, see
+                    // load_dword_from_row) and the shift that takes it out are found once per lane; a row's address is
+                    // the same for the whole wave.
+                    const unsigned base = static_cast<unsigned>(reinterpret_cast<size_t>(window));
+                    const unsigned off1 = static_cast<unsigned>(x1) * 3u, off2 = static_cast<unsigned>(x2) * 3u;
+                    const bool al1 = ((base + off1) & 3u) == 0u, al2 = ((base + off2) & 3u) == 0u;
+                    const unsigned voff1 = off1 + (al1 ? 1u : 0u), voff2 = off2 + (al2 ? 1u : 0u);
+                    const unsigned sh1 = al1 ? 0u : 8u, sh2 = al2 ? 0u : 8u;
+                    const auto pixel = [](const unsigned int w) {
+                        dev::PixelSlot<Src> px;
+                        px.w[0] = w;
+                        return to_tap(dev::slot_to_pixel<Src>(px));
+                    };
+                    for (int g = 0; g < wave_rows; g += RESIZE_GROUP_ROWS) {
+                        unsigned int a[RESIZE_GROUP_ROWS], b[RESIZE_GROUP_ROWS], c[RESIZE_GROUP_ROWS], d[RESIZE_GROUP_ROWS];
+#pragma unroll
+                        for (int k = 0; k < RESIZE_GROUP_ROWS; ++k) {
+                            const int ya = __builtin_amdgcn_readlane(y1, g + k), yb = __builtin_amdgcn_readlane(y2, g + k);
+                            const char* const r0 = window + static_cast<size_t>(ya) * s.pitch;
+                            const char* const r1 = window + static_cast<size_t>(yb) * s.pitch;
+                            a[k] = dev::load_dword_from_row(r0, voff1);
+                            b[k] = dev::load_dword_from_row(r0, voff2);
+                            c[k] = dev::load_dword_from_row(r1, voff1);
+                            d[k] = dev::load_dword_from_row(r1, voff2);
+                        }
+                        each_of_group([&](const auto k) {
+                            constexpr int K = decltype(k)::value;
+                            emit(g, k, pixel(a[K] >> sh1), pixel(b[K] >> sh2), pixel(c[K] >> sh1), pixel(d[K] >> sh2));
+                        });
+                    }
+                    return;
+                }
+            }
             for (int g = 0; g < wave_rows; g += RESIZE_GROUP_ROWS) {
                 Src a[RESIZE_GROUP_ROWS], b[RESIZE_GROUP_ROWS], c[RESIZE_GROUP_ROWS], d[RESIZE_GROUP_ROWS];
 #pragma unroll
@@ -907,62 +941,69 @@ struct ResizeJob {
             // staging pays off while a source pixel is used about once or more; strong down-scaling reads taps directly
             staged = (job.flags & FLAG_SOURCE_TILE) != 0u && rows * stride * SLOT <= static_cast<int>(job.tile_dwords) && rows * cols <= 3 * tile_px + 256;
             if (staged) {
-                // A wave takes every fourth row, a lane every 64th column; the loads of STAGE_ROWS rows are issued before
-                // the first of them is stored, so a tile of up to 4 * STAGE_ROWS rows costs one memory round trip.  A row
-                // past the tile's last is the last one again, loaded and stored twice: with a branch around it the
-                // compiler moves the load to the store and waits there.
+                // The lanes of a wave cover the box's columns, and where the box is narrow (32 columns or fewer) several
+                // of its rows side by side: lane = (row within the wave's pass, column).  The block's waves take the rows
+                // of a pass in turn.  Pixels read as they lie in memory (RAW_SOURCE): the loads of STAGE_ROWS passes are
+                // issued before the first of them is stored, so a box of up to STAGE_ROWS passes costs one memory round
+                // trip, and a row past the box's last is the last one again, loaded and stored twice (with a branch
+                // around it the compiler moves the load to the store and waits there).  Pixels that are computed
+                // (operations fused before the resize) are computed once each: lanes past the box's last row rest.
                 const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
                 constexpr int WAVES = BLOCK_THREADS / 64;
-                constexpr int STAGE_ROWS = sizeof(Src) <= 4 ? 4 : 2;
+                constexpr int STAGE_ROWS = RAW_SOURCE ? (sizeof(Src) <= 4 ? 4 : 2) : 2;
+                int lane_cols_log2 = 32 - __builtin_clz(static_cast<unsigned>(cols - 1)); // columns a wave puts side by side: >= cols, at most 64
+                lane_cols_log2 = lane_cols_log2 > 6 ? 6 : lane_cols_log2;
+                const int lane_cols = 1 << lane_cols_log2;
+                const int pass_rows = 64 >> lane_cols_log2;            // rows of a wave's pass
+                const int lane_row = wave * pass_rows + (lane >> lane_cols_log2); // this lane's row in the block's first pass
+                const int block_rows = WAVES * pass_rows;              // rows of a block's pass
                 bool rows_alike = false;
                 if constexpr (RAW_SOURCE && sizeof(Src) == 3) rows_alike = (s.pitch & 3u) == 0u;
-                if (rows_alike) {
+                for (int c = lane & (lane_cols - 1); c < cols; c += lane_cols) {
+                    const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
                     // three-byte pixels, rows a whole number of dwords apart: a column has the same alignment in every
                     // row, so a lane's offset and the shift that takes the pixel out of its dword are found once per column
-                    if constexpr (RAW_SOURCE && sizeof(Src) == 3) {
-                        for (int c = lane; c < cols; c += 64) {
-                            const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
-                            const unsigned off = static_cast<unsigned>(sx) * 3u;
-                            const bool aligned = ((static_cast<unsigned>(reinterpret_cast<size_t>(window)) + off) & 3u) == 0u;
-                            const unsigned voff = off + (aligned ? 1u : 0u); // from one byte before the row
-                            for (int r0 = wave; r0 < rows; r0 += WAVES * STAGE_ROWS) {
-                                unsigned int w[STAGE_ROWS];
+                    const unsigned off = static_cast<unsigned>(sx) * static_cast<unsigned>(sizeof(Src));
+                    const bool aligned = ((static_cast<unsigned>(reinterpret_cast<size_t>(window)) + off) & 3u) == 0u;
+                    const unsigned voff = off + (aligned ? 1u : 0u); // from one byte before the row
+                    for (int first = 0; first < rows; first += block_rows * STAGE_ROWS) { // (uniform)
+                        if constexpr (RAW_SOURCE) {
+                            dev::PixelSlot<Src> px[STAGE_ROWS];
 #pragma unroll
-                                for (int u = 0; u < STAGE_ROWS; ++u) {
-                                    const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
-                                    const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
-                                    w[u] = dev::load_dword_from_row(window + static_cast<size_t>(sy) * s.pitch, voff);
-                                }
-#pragma unroll
-                                for (int u = 0; u < STAGE_ROWS; ++u) {
-                                    const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
-                                    dev::PixelSlot<Src> px;
-                                    px.w[0] = aligned ? w[u] : w[u] >> 8u;
-                                    store_tap(tile + (r * stride + c) * SLOT, to_tap(dev::slot_to_pixel<Src>(px)));
+                            for (int u = 0; u < STAGE_ROWS; ++u) {
+                                const int wanted = first + block_rows * u + lane_row;
+                                const int r = wanted < rows ? wanted : rows - 1;
+                                const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
+                                if constexpr (sizeof(Src) == 3) {
+                                    // (a window of less than 2 GiB: the row's offset fits the lane's 32 bits)
+                                    if (rows_alike) {
+                                        const unsigned int w = dev::load_dword_from_row(window, static_cast<unsigned>(sy) * s.pitch + voff);
+                                        px[u].w[0] = aligned ? w : w >> 8u;
+                                    } else {
+                                        px[u] = dev::load_pixel_slot<Src>(window, static_cast<int>(static_cast<unsigned>(sy) * s.pitch + off), valid_lo, valid_hi);
+                                    }
+                                } else {
+                                    px[u] = dev::load_pixel_slot<Src>(window + static_cast<size_t>(sy) * s.pitch, static_cast<int>(off), valid_lo, valid_hi);
                                 }
                             }
-                        }
-                    }
-                } else
-                for (int c = lane; c < cols; c += 64) {
-                    const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
-                    for (int r0 = wave; r0 < rows; r0 += WAVES * STAGE_ROWS) {
-                        Src px[STAGE_ROWS];
 #pragma unroll
-                        for (int u = 0; u < STAGE_ROWS; ++u) {
-                            const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
-                            const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
-                            if constexpr (RAW_SOURCE) {
-                                const char* const row = window + static_cast<size_t>(sy) * s.pitch;
-                                px[u] = dev::slot_to_pixel<Src>(dev::load_pixel_slot<Src>(row, sx * static_cast<int>(sizeof(Src)), valid_lo, valid_hi));
-                            } else {
-                                px[u] = fetch(v, sx, sy);
+                            for (int u = 0; u < STAGE_ROWS; ++u) {
+                                const int wanted = first + block_rows * u + lane_row;
+                                const int r = wanted < rows ? wanted : rows - 1;
+                                store_tap(tile + (r * stride + c) * SLOT, to_tap(dev::slot_to_pixel<Src>(px[u])));
                             }
-                        }
+                        } else {
+                            Src px[STAGE_ROWS];
 #pragma unroll
-                        for (int u = 0; u < STAGE_ROWS; ++u) {
-                            const int r = r0 + WAVES * u < rows ? r0 + WAVES * u : rows - 1;
-                            store_tap(tile + (r * stride + c) * SLOT, to_tap(px[u]));
+                            for (int u = 0; u < STAGE_ROWS; ++u) {
+                                const int r = first + block_rows * u + lane_row;
+                                if (r < rows) px[u] = fetch(v, sx, sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1);
+                            }
+#pragma unroll
+                            for (int u = 0; u < STAGE_ROWS; ++u) {
+                                const int r = first + block_rows * u + lane_row;
+                                if (r < rows) store_tap(tile + (r * stride + c) * SLOT, to_tap(px[u]));
+                            }
                         }
                     }
                 }
