@@ -12,7 +12,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
 PRESERVE_AR, IGNORE_AR, PRESERVE_AR_RN_EVEN, PRESERVE_AR_LEFT = 0, 1, 2, 3
-BATCH_SIZES = (1, 2, 3, 5, 8, 32, 50)
+# (batches take any number of planes: it is a run-time value at the C boundary)
 CHAIN_DEPTHS = (1, 2, 4, 8, 16, 32, 64, 128)
 
 

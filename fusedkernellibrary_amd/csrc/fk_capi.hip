@@ -2,6 +2,7 @@
 // (PerThreadRead(...).then(...)..., TensorWrite) and hands it to executeOperations, which instantiates the fused
 // gfx950 kernel for that chain.  Compiled by hipcc into libfk_capi.so.
 #include <array>
+#include <vector>
 
 #include "fk_capi_common.h"
 
@@ -16,12 +17,7 @@ std::string& last_error() {
 } // namespace fk_capi
 
 namespace {
-template <size_t N>
-std::array<Rect, N> rects_of(const fk_rect* r) {
-    std::array<Rect, N> out;
-    for (size_t i = 0; i < N; ++i) out[i] = Rect(static_cast<uint>(r[i].x), static_cast<uint>(r[i].y), r[i].width, r[i].height);
-    return out;
-}
+Rect rect_of(const fk_rect& r) { return Rect(static_cast<uint>(r.x), static_cast<uint>(r.y), r.width, r.height); }
 float3 f3(const float* v) { return float3{ v[0], v[1], v[2] }; }
 
 bool rects_inside(const fk_rect* r, int n, int w, int h) {
@@ -33,68 +29,101 @@ bool rects_inside(const fk_rect* r, int n, int w, int h) {
 
 using Linear = InterpolationType;
 
-template <size_t N, AspectRatio AR>
-void readme_pipeline(Stream& stream, const void* src, int w, int h, size_t pitch, const fk_rect* rects, int dw, int dh,
-                     const float* bg, const float* mul, const float* sub, const float* div, float* out) {
-    const auto cropped = PerThreadRead<ND::_2D, uchar3>::build(view2d<uchar3>(src, w, h, pitch)).then(Crop<>::build(rects_of<N>(rects)));
-    const auto receiver = TensorWrite<float3>::build(view3d<float3>(out, dw, dh, static_cast<int>(N), 1));
-    const auto finish = [&](const auto& resized) {
-        const auto sender = resized.then(Mul<float3>::build(f3(mul)))
-                                .then(Sub<float3>::build(f3(sub)))
-                                .then(Div<float3>::build(f3(div)))
-                                .then(ColorConversion<ColorConversionCodes::COLOR_RGB2BGR, float3, float3>::build());
-        executeOperations<TransformDPP<>>(stream, sender, receiver);
-    };
-    if constexpr (AR == AspectRatio::IGNORE_AR) {
-        finish(cropped.then(Resize<Linear::INTER_LINEAR, AR>::build(Size(dw, dh))));
-    } else {
-        finish(cropped.then(Resize<Linear::INTER_LINEAR, AR>::build(Size(dw, dh), f3(bg))));
+// A batch of n planes, n known at run time: the planes are built one by one with the same .then() chain (what the
+// batch builders of the operator API do per element of their arrays), put into batch reads of a fixed capacity with n of
+// their entries in use, and launched 64 planes at a time; `receiver_for(first, count)` builds the write for planes
+// first .. first + count - 1.  The plane table travels in the kernel-argument segment like that of a batch whose size is
+// a template argument.
+constexpr size_t SMALL_BATCH = 8, LARGE_BATCH = 64;
+template <typename PlaneIOp, typename ReceiverFor>
+void launch_planes(Stream& stream, const std::vector<PlaneIOp>& planes, const ReceiverFor& receiver_for) {
+    for (size_t first = 0; first < planes.size(); first += LARGE_BATCH) {
+        const size_t count = planes.size() - first < LARGE_BATCH ? planes.size() - first : LARGE_BATCH;
+        if (count <= SMALL_BATCH) {
+            executeOperations<TransformDPP<>>(stream, BatchRead<SMALL_BATCH>::build_first(&planes[first], count), receiver_for(first, count));
+        } else {
+            executeOperations<TransformDPP<>>(stream, BatchRead<LARGE_BATCH>::build_first(&planes[first], count), receiver_for(first, count));
+        }
     }
 }
 
-template <size_t N>
-int readme_pipeline_any_ar(Stream& stream, int aspect, const void* src, int w, int h, size_t pitch, const fk_rect* rects, int dw,
+template <AspectRatio AR>
+void readme_pipeline(Stream& stream, const void* src, int w, int h, size_t pitch, const fk_rect* rects, int n, int dw, int dh,
+                     const float* bg, const float* mul, const float* sub, const float* div, float* out) {
+    const auto read = PerThreadRead<ND::_2D, uchar3>::build(view2d<uchar3>(src, w, h, pitch));
+    const auto plane = [&](const fk_rect& r) {
+        const auto cropped = read.then(Crop<>::build(rect_of(r)));
+        const auto finish = [&](const auto& resized) {
+            return resized.then(Mul<float3>::build(f3(mul)))
+                .then(Sub<float3>::build(f3(sub)))
+                .then(Div<float3>::build(f3(div)))
+                .then(ColorConversion<ColorConversionCodes::COLOR_RGB2BGR, float3, float3>::build());
+        };
+        if constexpr (AR == AspectRatio::IGNORE_AR) {
+            return finish(cropped.then(Resize<Linear::INTER_LINEAR, AR>::build(Size(dw, dh))));
+        } else {
+            return finish(cropped.then(Resize<Linear::INTER_LINEAR, AR>::build(Size(dw, dh), f3(bg))));
+        }
+    };
+    std::vector<decltype(plane(rects[0]))> planes;
+    for (int i = 0; i < n; ++i) planes.push_back(plane(rects[i]));
+    const size_t plane_floats = static_cast<size_t>(dw) * dh * 3;
+    launch_planes(stream, planes, [&](size_t first, size_t count) {
+        return TensorWrite<float3>::build(view3d<float3>(out + first * plane_floats, dw, dh, static_cast<int>(count), 1));
+    });
+}
+
+int readme_pipeline_any_ar(Stream& stream, int aspect, const void* src, int w, int h, size_t pitch, const fk_rect* rects, int n, int dw,
                            int dh, const float* bg, const float* mul, const float* sub, const float* div, float* out) {
     switch (aspect) {
-    case FK_PRESERVE_AR: readme_pipeline<N, AspectRatio::PRESERVE_AR>(stream, src, w, h, pitch, rects, dw, dh, bg, mul, sub, div, out); return FK_OK;
-    case FK_IGNORE_AR: readme_pipeline<N, AspectRatio::IGNORE_AR>(stream, src, w, h, pitch, rects, dw, dh, bg, mul, sub, div, out); return FK_OK;
-    case FK_PRESERVE_AR_RN_EVEN: readme_pipeline<N, AspectRatio::PRESERVE_AR_RN_EVEN>(stream, src, w, h, pitch, rects, dw, dh, bg, mul, sub, div, out); return FK_OK;
-    case FK_PRESERVE_AR_LEFT: readme_pipeline<N, AspectRatio::PRESERVE_AR_LEFT>(stream, src, w, h, pitch, rects, dw, dh, bg, mul, sub, div, out); return FK_OK;
+    case FK_PRESERVE_AR: readme_pipeline<AspectRatio::PRESERVE_AR>(stream, src, w, h, pitch, rects, n, dw, dh, bg, mul, sub, div, out); return FK_OK;
+    case FK_IGNORE_AR: readme_pipeline<AspectRatio::IGNORE_AR>(stream, src, w, h, pitch, rects, n, dw, dh, bg, mul, sub, div, out); return FK_OK;
+    case FK_PRESERVE_AR_RN_EVEN: readme_pipeline<AspectRatio::PRESERVE_AR_RN_EVEN>(stream, src, w, h, pitch, rects, n, dw, dh, bg, mul, sub, div, out); return FK_OK;
+    case FK_PRESERVE_AR_LEFT: readme_pipeline<AspectRatio::PRESERVE_AR_LEFT>(stream, src, w, h, pitch, rects, n, dw, dh, bg, mul, sub, div, out); return FK_OK;
     default: return unsupported("unknown aspect-ratio mode");
     }
 }
 
-template <size_t N>
-void split_pipeline(Stream& stream, const void* const* srcs, int w, int h, size_t pitch, const fk_rect* rects, int dw, int dh,
+void split_pipeline(Stream& stream, const void* const* srcs, int w, int h, size_t pitch, const fk_rect* rects, int n, int dw, int dh,
                     const float* d1, const float* s, const float* d2, float* out) {
-    std::array<RawPtr<ND::_2D, uchar3>, N> images;
-    for (size_t i = 0; i < N; ++i) images[i] = view2d<uchar3>(srcs[i], w, h, pitch);
-    const auto sender = PerThreadRead<ND::_2D, uchar3>::build(images)
-                            .then(Crop<>::build(rects_of<N>(rects)))
-                            .then(Resize<Linear::INTER_LINEAR>::build(Size(dw, dh)))
-                            .then(Div<float3>::build(f3(d1)))
-                            .then(Sub<float3>::build(f3(s)))
-                            .then(Div<float3>::build(f3(d2)))
-                            .then(ColorConversion<ColorConversionCodes::COLOR_RGB2BGR, float3, float3>::build());
-    executeOperations<TransformDPP<>>(stream, sender, TensorSplit<float3>::build(view3d<float>(out, dw, dh, static_cast<int>(N), 3)));
+    const auto plane = [&](const void* src, const fk_rect& r) {
+        return PerThreadRead<ND::_2D, uchar3>::build(view2d<uchar3>(src, w, h, pitch))
+            .then(Crop<>::build(rect_of(r)))
+            .then(Resize<Linear::INTER_LINEAR>::build(Size(dw, dh)))
+            .then(Div<float3>::build(f3(d1)))
+            .then(Sub<float3>::build(f3(s)))
+            .then(Div<float3>::build(f3(d2)))
+            .then(ColorConversion<ColorConversionCodes::COLOR_RGB2BGR, float3, float3>::build());
+    };
+    std::vector<decltype(plane(srcs[0], rects[0]))> planes;
+    for (int i = 0; i < n; ++i) planes.push_back(plane(srcs[i], rects[i]));
+    const size_t plane_floats = static_cast<size_t>(dw) * dh * 3;
+    launch_planes(stream, planes, [&](size_t first, size_t count) {
+        return TensorSplit<float3>::build(view3d<float>(out + first * plane_floats, dw, dh, static_cast<int>(count), 3));
+    });
 }
 
-template <size_t N>
-void tiles_pipeline(Stream& stream, const void* src, int w, int h, size_t pitch, int rw, int rh, const fk_rect* rects, int tw,
+void tiles_pipeline(Stream& stream, const void* src, int w, int h, size_t pitch, int rw, int rh, const fk_rect* rects, int n, int tw,
                     int th, const float* mul, float* out) {
-    const auto sender = PerThreadRead<ND::_2D, uchar3>::build(view2d<uchar3>(src, w, h, pitch))
-                            .then(Resize<Linear::INTER_LINEAR>::build(Size(rw, rh)))
-                            .then(Crop<>::build(rects_of<N>(rects)))
-                            .then(Mul<float3>::build(f3(mul)));
-    executeOperations<TransformDPP<>>(stream, sender, TensorWrite<float3>::build(view3d<float3>(out, tw, th, static_cast<int>(N), 1)));
+    const auto resized = PerThreadRead<ND::_2D, uchar3>::build(view2d<uchar3>(src, w, h, pitch)).then(Resize<Linear::INTER_LINEAR>::build(Size(rw, rh)));
+    const auto plane = [&](const fk_rect& r) { return resized.then(Crop<>::build(rect_of(r))).then(Mul<float3>::build(f3(mul))); };
+    std::vector<decltype(plane(rects[0]))> planes;
+    for (int i = 0; i < n; ++i) planes.push_back(plane(rects[i]));
+    const size_t plane_floats = static_cast<size_t>(tw) * th * 3;
+    launch_planes(stream, planes, [&](size_t first, size_t count) {
+        return TensorWrite<float3>::build(view3d<float3>(out + first * plane_floats, tw, th, static_cast<int>(count), 1));
+    });
 }
 
-template <size_t N>
-void crops_pipeline(Stream& stream, const void* src, int w, int h, size_t pitch, const fk_rect* rects, int mw, int mh, float* out) {
-    const auto sender = PerThreadRead<ND::_2D, uchar3>::build(view2d<uchar3>(src, w, h, pitch))
-                            .then(Crop<>::build(rects_of<N>(rects)))
-                            .then(Cast<uchar3, float3>::build());
-    executeOperations<TransformDPP<>>(stream, sender, TensorWrite<float3>::build(view3d<float3>(out, mw, mh, static_cast<int>(N), 1)));
+void crops_pipeline(Stream& stream, const void* src, int w, int h, size_t pitch, const fk_rect* rects, int n, int mw, int mh, float* out) {
+    const auto read = PerThreadRead<ND::_2D, uchar3>::build(view2d<uchar3>(src, w, h, pitch));
+    const auto plane = [&](const fk_rect& r) { return read.then(Crop<>::build(rect_of(r))).then(Cast<uchar3, float3>::build()); };
+    std::vector<decltype(plane(rects[0]))> planes;
+    for (int i = 0; i < n; ++i) planes.push_back(plane(rects[i]));
+    const size_t plane_floats = static_cast<size_t>(mw) * mh * 3;
+    launch_planes(stream, planes, [&](size_t first, size_t count) {
+        return TensorWrite<float3>::build(view3d<float3>(out + first * plane_floats, mw, mh, static_cast<int>(count), 1));
+    });
 }
 
 // read -> Mul -> Add -> Mul -> ... (DEPTH operations) -> write, built one .then() at a time
@@ -139,18 +168,6 @@ void run_sequence(Stream& stream, const Sequence& seq) {
 }
 } // namespace
 
-#define FK_FOR_BATCH(n, CALL)                                                                                          \
-    switch (n) {                                                                                                       \
-    case 1: { constexpr size_t N = 1; CALL; break; }                                                                   \
-    case 2: { constexpr size_t N = 2; CALL; break; }                                                                   \
-    case 3: { constexpr size_t N = 3; CALL; break; }                                                                   \
-    case 5: { constexpr size_t N = 5; CALL; break; }                                                                   \
-    case 8: { constexpr size_t N = 8; CALL; break; }                                                                   \
-    case 32: { constexpr size_t N = 32; CALL; break; }                                                                 \
-    case 50: { constexpr size_t N = 50; CALL; break; }                                                                 \
-    default: return unsupported("batch size has no instantiation (1, 2, 3, 5, 8, 32, 50)");                            \
-    }
-
 extern "C" {
 
 const char* fk_last_error(void) { return last_error().c_str(); }
@@ -166,13 +183,11 @@ int fk_interpolate_y1_from_x(void) {
 int fk_crop_resize_muls_bgr_tensor(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n, int dst_w,
                                    int dst_h, int aspect, const float background[3], const float mul[3], const float sub[3],
                                    const float div[3], float* out, void* stream) {
-    if (src == nullptr || out == nullptr || rects == nullptr || dst_w <= 0 || dst_h <= 0) return bad_argument("null pointer or empty destination");
+    if (src == nullptr || out == nullptr || rects == nullptr || dst_w <= 0 || dst_h <= 0 || n <= 0) return bad_argument("null pointer, empty destination or no planes");
     if (!rects_inside(rects, n, src_w, src_h)) return bad_argument("crop rectangle outside the source image");
     return guarded([&]() -> int {
         Stream s(stream);
-        int rc = FK_OK;
-        FK_FOR_BATCH(n, (rc = readme_pipeline_any_ar<N>(s, aspect, src, src_w, src_h, src_pitch, rects, dst_w, dst_h, background, mul, sub, div, out)))
-        return rc;
+        return readme_pipeline_any_ar(s, aspect, src, src_w, src_h, src_pitch, rects, n, dst_w, dst_h, background, mul, sub, div, out);
     });
 }
 
@@ -213,25 +228,25 @@ int fk_single_op_f32c3(const void* src, int w, int h, size_t src_pitch, int is_a
 int fk_batch_crop_resize_norm_split(const void* const* srcs, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n,
                                     int dst_w, int dst_h, const float div1[3], const float sub[3], const float div2[3], float* out,
                                     void* stream) {
-    if (srcs == nullptr || out == nullptr || rects == nullptr || dst_w <= 0 || dst_h <= 0) return bad_argument("null pointer or empty destination");
+    if (srcs == nullptr || out == nullptr || rects == nullptr || dst_w <= 0 || dst_h <= 0 || n <= 0) return bad_argument("null pointer, empty destination or no planes");
     if (!rects_inside(rects, n, src_w, src_h)) return bad_argument("crop rectangle outside the source image");
     return guarded([&]() -> int {
         Stream s(stream);
-        FK_FOR_BATCH(n, (split_pipeline<N>(s, srcs, src_w, src_h, src_pitch, rects, dst_w, dst_h, div1, sub, div2, out)))
+        split_pipeline(s, srcs, src_w, src_h, src_pitch, rects, n, dst_w, dst_h, div1, sub, div2, out);
         return FK_OK;
     });
 }
 
 int fk_resize_crop_tiles(const void* src, int src_w, int src_h, size_t src_pitch, int rs_w, int rs_h, const fk_rect* rects, int n,
                          int tile_w, int tile_h, const float mul[3], float* out, void* stream) {
-    if (src == nullptr || out == nullptr || rects == nullptr || rs_w <= 0 || rs_h <= 0) return bad_argument("null pointer or empty destination");
+    if (src == nullptr || out == nullptr || rects == nullptr || rs_w <= 0 || rs_h <= 0 || n <= 0) return bad_argument("null pointer, empty destination or no planes");
     if (!rects_inside(rects, n, rs_w, rs_h)) return bad_argument("tile outside the resized image");
     for (int i = 0; i < n; ++i) {
         if (rects[i].width != tile_w || rects[i].height != tile_h) return bad_argument("every tile must be tile_w x tile_h");
     }
     return guarded([&]() -> int {
         Stream s(stream);
-        FK_FOR_BATCH(n, (tiles_pipeline<N>(s, src, src_w, src_h, src_pitch, rs_w, rs_h, rects, tile_w, tile_h, mul, out)))
+        tiles_pipeline(s, src, src_w, src_h, src_pitch, rs_w, rs_h, rects, n, tile_w, tile_h, mul, out);
         return FK_OK;
     });
 }
@@ -292,14 +307,14 @@ int fk_divergent4_u8c4(const void* src, int w, int h, size_t src_pitch, void* gr
 
 int fk_batch_crop_cast_tensor(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n, int max_w,
                               int max_h, float* out, void* stream) {
-    if (src == nullptr || out == nullptr || rects == nullptr) return bad_argument("null pointer");
+    if (src == nullptr || out == nullptr || rects == nullptr || n <= 0) return bad_argument("null pointer or no planes");
     if (!rects_inside(rects, n, src_w, src_h)) return bad_argument("crop rectangle outside the source image");
     for (int i = 0; i < n; ++i) {
         if (rects[i].width > max_w || rects[i].height > max_h) return bad_argument("crop larger than the tensor plane");
     }
     return guarded([&]() -> int {
         Stream s(stream);
-        FK_FOR_BATCH(n, (crops_pipeline<N>(s, src, src_w, src_h, src_pitch, rects, max_w, max_h, out)))
+        crops_pipeline(s, src, src_w, src_h, src_pitch, rects, n, max_w, max_h, out);
         return FK_OK;
     });
 }

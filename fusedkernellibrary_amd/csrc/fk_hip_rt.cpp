@@ -24,12 +24,6 @@ extern "C" {
 int fkrt_device_count(int* count) { return static_cast<int>(hipGetDeviceCount(count)); }
 int fkrt_set_device(int device) { return static_cast<int>(hipSetDevice(device)); }
 int fkrt_get_device(int* device) { return static_cast<int>(hipGetDevice(device)); }
-int fkrt_device_compute_units(int* count) {
-    int device = 0;
-    hipError_t e = hipGetDevice(&device);
-    if (e != hipSuccess) return static_cast<int>(e);
-    return static_cast<int>(hipDeviceGetAttribute(count, hipDeviceAttributeMultiprocessorCount, device));
-}
 
 int fkrt_stream_create(fkrt_stream* out) {
     hipStream_t s = nullptr;

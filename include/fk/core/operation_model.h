@@ -688,6 +688,29 @@ struct BatchRead<BATCH_, PP_, void, NullType> {
         return Batch::build(params);
     }
 
+    // A batch whose number of planes is known only at run time (this library's extension: the reference fixes it with
+    // BATCH, batch_operations.h:153-208): the first `count` entries of a table of BATCH planes are filled in, and the
+    // batch's thread grid has `count` planes.
+    template <typename IOp>
+    static inline auto build_first(const IOp* iOps, size_t count) {
+        static_assert(PP_ == PlanePolicy::PROCESS_ALL, "every plane of a run-time batch is processed");
+        static_assert(isAnyReadType<IOp>, "BatchRead is made of Read or ReadBack operations");
+        using Op = typename IOp::Operation;
+        using Batch = BatchRead<BATCH_, PlanePolicy::PROCESS_ALL, Op>;
+        typename Batch::ParamsType params{};
+        count = count < BATCH_ ? count : BATCH_;
+        uint max_w = 0, max_h = 0;
+        for (size_t i = 0; i < count; ++i) {
+            params.opData[i] = static_cast<const OperationData<Op>&>(iOps[i]);
+            const uint w = Op::num_elems_x(Point(0, 0, 0), iOps[i]);
+            const uint h = Op::num_elems_y(Point(0, 0, 0), iOps[i]);
+            max_w = w > max_w ? w : max_w;
+            max_h = h > max_h ? h : max_h;
+        }
+        params.activeThreads = ActiveThreads(max_w, max_h, static_cast<uint>(count));
+        return Batch::build(params);
+    }
+
 private:
     template <typename Params, typename IOp>
     static inline constexpr void fill(Params& params, const std::array<IOp, BATCH_>& iOps) {

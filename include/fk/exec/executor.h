@@ -65,20 +65,37 @@ inline unsigned resize_wave_rows_override() {
 
 // ---- job construction ----------------------------------------------------------------------------------------
 namespace detail {
+// The planes of a sender: `capacity` is the size of its plane table (known at compile time), `count` the planes of the
+// thread grid (a batch filled in at run time holds fewer than its capacity), `used` the planes that run their program
+// (the others receive the default value of a CONDITIONAL_WITH_DEFAULT batch).
 template <typename Sender, typename = void>
 struct PlaneIOpOf {
     using type = Sender;
-    static constexpr size_t planes = 1;
-    static constexpr bool process_all = true;
+    static constexpr size_t capacity = 1;
+    static constexpr bool conditional = false;
     static const type& get(const Sender& s, size_t) { return s; }
+    static size_t count(const Sender&) { return 1; }
+    static size_t used(const Sender&) { return 1; }
 };
 template <typename Sender>
 struct PlaneIOpOf<Sender, std::enable_if_t<isBatchOperation<typename Sender::Operation>>> {
     using Batch = typename Sender::Operation;
     using type = Instantiable<typename Batch::Operation>;
-    static constexpr size_t planes = Batch::BATCH;
-    static constexpr bool process_all = Batch::PP == PlanePolicy::PROCESS_ALL;
+    static constexpr size_t capacity = Batch::BATCH;
+    static constexpr bool conditional = Batch::PP == PlanePolicy::CONDITIONAL_WITH_DEFAULT;
     static type get(const Sender& s, size_t i) { return toIOp<typename Batch::Operation>(s.params.opData[i]); }
+    static size_t count(const Sender& s) {
+        const size_t z = s.params.activeThreads.z;
+        return z < capacity ? z : capacity;
+    }
+    static size_t used(const Sender& s) {
+        if constexpr (conditional) {
+            const size_t n = count(s), u = s.params.usedPlanes < 0 ? 0 : static_cast<size_t>(s.params.usedPlanes);
+            return u < n ? u : n;
+        } else {
+            return count(s);
+        }
+    }
 };
 template <typename PlaneIOp, typename = void>
 struct IsResizeProgram : std::false_type {};
@@ -96,7 +113,7 @@ template <typename Sender, typename Receiver>
 struct JobOf {
     using Planes = detail::PlaneIOpOf<Sender>;
     using PlaneIOp = typename Planes::type;
-    static constexpr size_t N = Planes::planes;
+    static constexpr size_t N = Planes::capacity;
 #ifdef FK_INTERPOLATE_Y1_FROM_X
     // the reference's host-branch interpolation takes the tap row from the x coordinate: rows and columns are no longer
     // separable, so resize chains run on the generic per-element kernel in such a build
@@ -104,18 +121,39 @@ struct JobOf {
 #else
     static constexpr bool separable = true;
 #endif
-    static constexpr bool viewable = Planes::process_all && separable && detail::Matches<PlaneIOp, Receiver>::value;
+    static constexpr bool viewable = separable && detail::Matches<PlaneIOp, Receiver>::value;
+
+    // what the planes from `used` on receive (a CONDITIONAL_WITH_DEFAULT batch), with the extent of the batch's grid
+    template <typename Defaults>
+    static Defaults defaults_of(const Sender& sender) {
+        if constexpr (Defaults::ENABLED) {
+            const ActiveThreads grid = sender.getActiveThreads();
+            return Defaults{ static_cast<unsigned>(Planes::used(sender)), static_cast<int>(grid.x), static_cast<int>(grid.y), sender.params.default_value };
+        } else {
+            return Defaults{};
+        }
+    }
 
     static auto make(const Sender& sender, const Receiver& receiver) {
         if constexpr (viewable) {
             using Prog = typename ProgramOf<PlaneIOp>::type;
             using Out = typename OutOf<Receiver>::type;
             using View = decltype(Prog::view);
+            using Defaults = std::conditional_t<Planes::conditional, DefaultPlanes<typename Out::Pixel>, NoDefaultPlanes>;
             const Out out = OutOf<Receiver>::make(receiver);
+            const size_t count = Planes::count(sender), used = Planes::used(sender);
+            const Defaults defaults = defaults_of<Defaults>(sender);
+            int max_w = 0, max_h = 0;
+            if constexpr (Defaults::ENABLED) {
+                if (used < count) {
+                    max_w = defaults.w;
+                    max_h = defaults.h;
+                }
+            }
             if constexpr (View::IS_RESIZE) {
-                ResizeJob<Prog, N, Out> job{};
-                int max_w = 0, max_h = 0;
-                for (size_t i = 0; i < N; ++i) {
+                ResizeJob<Prog, N, Out, Defaults> job{};
+                job.defaults = defaults;
+                for (size_t i = 0; i < used; ++i) {
                     job.plane[i] = ProgramOf<PlaneIOp>::make(Planes::get(sender, i));
                     max_w = job.plane[i].view.w > max_w ? job.plane[i].view.w : max_w;
                     max_h = job.plane[i].view.h > max_h ? job.plane[i].view.h : max_h;
@@ -127,22 +165,22 @@ struct JobOf {
                 // (the kernel addresses a wave's rows, and their channel planes, with 32-bit offsets from its first row)
                 if constexpr (Out::IS_SPLIT) dwords = dwords && out.chan_stride % 4 == 0 && out.chan_stride * 4 + static_cast<size_t>(out.pitch) * 64 < (1u << 30);
                 dwords = dwords && static_cast<size_t>(out.pitch) * 64 < (1u << 30);
-                const bool large = static_cast<size_t>(max_w) * max_h * N * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
+                const bool large = static_cast<size_t>(max_w) * max_h * count * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
                 job.flags = dwords && large ? FLAG_STREAM_STORES : 0u;
                 // tile height, grid rows and LDS layout; sets FLAG_SOURCE_TILE when some plane's tiles are worth staging
-                job.grid_y = job.plan(max_h, resize_wave_rows_override());
+                job.grid_y = job.plan(used, max_h, resize_wave_rows_override());
                 return job;
             } else {
-                using Job = PointwiseJob<Prog, N, Out>;
+                using Job = PointwiseJob<Prog, N, Out, Defaults>;
                 using Src = typename Job::Src;
                 using Access = typename Job::Access;
                 Job job{};
+                job.defaults = defaults;
                 job.out = out;
                 constexpr size_t out_elem = Out::IS_SPLIT ? sizeof(VBase<typename Out::Pixel>) : sizeof(typename Out::Pixel);
                 constexpr size_t out_chunk = dev::chunk_bytes(Job::K * static_cast<int>(out_elem));
-                int max_w = 0, max_h = 0;
-                bool flatten = Access::FLATTENS;
-                for (size_t i = 0; i < N; ++i) {
+                bool flatten = Access::FLATTENS && used == count;
+                for (size_t i = 0; i < used; ++i) {
                     job.plane[i].prog = ProgramOf<PlaneIOp>::make(Planes::get(sender, i));
                     if constexpr (Access::FLATTENS) {
                         const auto& v = job.plane[i].prog.view;
@@ -151,7 +189,7 @@ struct JobOf {
                                   static_cast<size_t>(v.w) * v.h < (1u << 30);
                     }
                 }
-                for (size_t i = 0; i < N; ++i) {
+                for (size_t i = 0; i < used; ++i) {
                     auto& v = job.plane[i].prog.view;
                     if constexpr (Access::FLATTENS) {
                         if (flatten) {
@@ -166,7 +204,7 @@ struct JobOf {
                     vec = vec && aligned_to(ofirst, out_chunk) && (v.h == 1 || out.pitch % out_chunk == 0);
                     if constexpr (Out::IS_SPLIT) vec = vec && out.chan_stride % out_chunk == 0;
                     // outputs larger than the caches are written with streaming stores
-                    const bool stream = static_cast<size_t>(v.w) * v.h * N * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
+                    const bool stream = static_cast<size_t>(v.w) * v.h * count * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
                     job.plane[i].flags = (vec ? FLAG_VECTOR_IO : 0u) | (vec && stream ? FLAG_STREAM_STORES : 0u);
                     max_w = v.w > max_w ? v.w : max_w;
                     max_h = v.h > max_h ? v.h : max_h;
@@ -220,7 +258,7 @@ struct JobOf {
         }
     }
     static unsigned planes(const Sender& sender) {
-        if constexpr (viewable) return static_cast<unsigned>(N);
+        if constexpr (viewable) return static_cast<unsigned>(Planes::count(sender));
         else return sender.getActiveThreads().z;
     }
 };

@@ -426,10 +426,33 @@ struct SourceAccess<YuvView<PF>> {
     }
 };
 
+// ---- planes that only receive a value ----------------------------------------------------------------------------
+// A batch read with PlanePolicy::CONDITIONAL_WITH_DEFAULT yields its default value for every element of the planes from
+// `used` on (reference batch_operations.h:234-241); those planes have the extent of the batch's thread grid.  A job of
+// such a batch carries this, and its blocks of those planes write the value and nothing else.
+template <typename O>
+struct DefaultPlanes {
+    static constexpr bool ENABLED = true;
+    unsigned used; // planes that run their program; the rest receive `value`
+    int w, h;      // extent of the planes that receive the value
+    O value;
+};
+struct NoDefaultPlanes {
+    static constexpr bool ENABLED = false;
+};
+namespace dev {
+// the part of such a plane that lies in columns x0 .. x0 + nx - 1 of row y, written by one thread
+template <typename Out, typename O>
+__device__ __attribute__((always_inline)) inline void fill_default(const Out& out, const DefaultPlanes<O>& d, int x0, int nx, int y, int z) {
+    if (y >= d.h) return;
+    for (int x = x0; x < x0 + nx && x < d.w; ++x) store_one(out, x, y, z, d.value);
+}
+} // namespace dev
+
 // ---- pointwise ---------------------------------------------------------------------------------------------------
 enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u };
 
-template <typename Prog, size_t N, typename Out>
+template <typename Prog, size_t N, typename Out, typename Defaults = NoDefaultPlanes>
 struct PointwiseJob {
     using View = decltype(Prog::view);
     using Access = SourceAccess<View>;
@@ -458,6 +481,7 @@ struct PointwiseJob {
     unsigned tx_shift; // log2 of the thread columns of a block; the other threads cover further rows
     unsigned grid_x, grid_y;
     unsigned pair_limit; // blocks that are re-dealt so that row pairs share an XCD (0: none)
+    Defaults defaults;
     size_t lds_bytes() const { return LDS_BYTES; }
 
     // A block that lies on one row and owns `span` pixels of it from pixel bx0 on (a whole number of thread groups, so
@@ -533,6 +557,14 @@ struct PointwiseJob {
     }
 
     __device__ __attribute__((always_inline)) static inline void run(const PointwiseJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char* lds) {
+        if constexpr (Defaults::ENABLED) {
+            if (bz >= job.defaults.used) {
+                const int cols = 1 << job.tx_shift, t = dev::thread_in_block();
+                dev::fill_default(job.out, job.defaults, (static_cast<int>(bx) * cols + (t & (cols - 1))) * K, K,
+                                  static_cast<int>(by) * (BLOCK_THREADS >> job.tx_shift) + (t >> job.tx_shift), static_cast<int>(bz));
+                return;
+            }
+        }
         const Plane& pl = job.plane[N == 1 ? 0u : bz];
         const View& v = pl.prog.view;
         const int tid = dev::thread_in_block();
@@ -665,7 +697,7 @@ __device__ __attribute__((always_inline)) inline PixelSlot<T> load_pixel_slot(co
 }
 } // namespace dev
 
-template <typename Prog, size_t N, typename Out>
+template <typename Prog, size_t N, typename Out, typename Defaults = NoDefaultPlanes>
 struct ResizeJob {
     using View = decltype(Prog::view);
     using SrcView = decltype(View::src);
@@ -698,6 +730,7 @@ struct ResizeJob {
     // The launch asks for as much LDS as the planes' own factors need, not for the capacity: a block's LDS decides how
     // many blocks a CU holds.  tile_dwords is the room for a source tile (a tile that needs more reads its taps directly).
     unsigned tile_dwords;
+    Defaults defaults;
     size_t lds_bytes() const { return (flags & FLAG_SOURCE_TILE) != 0u ? static_cast<size_t>(tile_dwords) * 4 + 16 : 0; }
     int tile_h() const { return (BLOCK_THREADS / 64) * static_cast<int>(wave_rows); }
     // dwords a tile of a plane with these factors takes when staged, 0 when it is not worth staging (same rule as the
@@ -710,15 +743,15 @@ struct ResizeJob {
         const bool worth = rows * (cols | 1) * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * RESIZE_TILE_W * tile_h + 256;
         return worth ? static_cast<unsigned>(rows * (cols | 1) * SLOT) : 0u;
     }
-    // Chooses the tile height and the LDS size from the planes' factors; grid_x has been decided, max_h is the tallest
-    // plane.  Returns the number of tile rows (grid_y).
-    unsigned plan(int max_h, unsigned forced_wave_rows) {
+    // Chooses the tile height and the LDS size from the factors of the first `count` planes; grid_x has been decided,
+    // max_h is the tallest plane.  Returns the number of tile rows (grid_y).
+    unsigned plan(size_t count, int max_h, unsigned forced_wave_rows) {
         // the tallest tile that still leaves the grid enough blocks, and whose source boxes fit the LDS wherever those of
         // the smallest tile do
-        const auto blocks = [&](unsigned wr) { return static_cast<size_t>(N) * grid_x * ((static_cast<unsigned>(max_h) + 4u * wr - 1u) / (4u * wr)); };
+        const auto blocks = [&](unsigned wr) { return count * grid_x * ((static_cast<unsigned>(max_h) + 4u * wr - 1u) / (4u * wr)); };
         const auto staged_planes = [&](unsigned wr) {
             unsigned n = 0;
-            for (size_t i = 0; i < N; ++i) n += staged_tile_dwords(plane[i].view.fx, plane[i].view.fy, 4 * static_cast<int>(wr)) != 0u ? 1u : 0u;
+            for (size_t i = 0; i < count; ++i) n += staged_tile_dwords(plane[i].view.fx, plane[i].view.fy, 4 * static_cast<int>(wr)) != 0u ? 1u : 0u;
             return n;
         };
         wave_rows = RESIZE_GROUP_ROWS;
@@ -726,7 +759,7 @@ struct ResizeJob {
         else if (blocks(8) >= RESIZE_MIN_BLOCKS_8 && staged_planes(8) == staged_planes(RESIZE_GROUP_ROWS)) wave_rows = 8;
         if (forced_wave_rows == 4u || forced_wave_rows == 8u || forced_wave_rows == 16u) wave_rows = forced_wave_rows;
         tile_dwords = 0;
-        for (size_t i = 0; i < N; ++i) {
+        for (size_t i = 0; i < count; ++i) {
             const unsigned need = staged_tile_dwords(plane[i].view.fx, plane[i].view.fy, tile_h());
             tile_dwords = need > tile_dwords ? need : tile_dwords;
         }
@@ -899,6 +932,16 @@ struct ResizeJob {
     }
 
     __device__ __attribute__((always_inline)) static inline void run(const ResizeJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char* lds_raw) {
+        if constexpr (Defaults::ENABLED) {
+            if (bz >= job.defaults.used) {
+                const int t = dev::thread_in_block(), rows = static_cast<int>(job.wave_rows);
+                const int y0 = (static_cast<int>(by) * (BLOCK_THREADS / 64) + (t >> 6)) * rows;
+                for (int i = 0; i < rows; ++i) {
+                    dev::fill_default(job.out, job.defaults, static_cast<int>(bx) * RESIZE_TILE_W + (t & 63), 1, y0 + i, static_cast<int>(bz));
+                }
+                return;
+            }
+        }
         const Prog& prog = job.plane[N == 1 ? 0u : bz];
         const View& v = prog.view;
         const SrcView& s = v.src;

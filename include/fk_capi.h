@@ -4,7 +4,7 @@
  * below is one such chain, instantiated from this library's fk:: templates (include/fk/) for a caller that cannot
  * compile templates (ctypes, cgo, JNI ...).  Device pointers and sizes only; `stream` is a hipStream_t (NULL = default
  * stream); work is enqueued asynchronously, the caller synchronises the stream.  Return value: 0 = enqueued,
- * FK_ERR_UNSUPPORTED = the batch size / depth / mode has no instantiation, FK_ERR_RUNTIME = the GPU runtime reported
+ * FK_ERR_UNSUPPORTED = the depth / format / mode has no instantiation, FK_ERR_RUNTIME = the GPU runtime reported
  * an error (text from fk_last_error()), FK_ERR_ARGUMENT = inconsistent arguments.
  *
  * Reference interface each one stands for (paths below the reference's include/fused_kernel/ unless noted):
@@ -39,7 +39,9 @@ int fk_interpolate_y1_from_x(void);
 /* The README pipeline (tests/examples/readme_test_code.h:26-72 of the reference):
  * PerThreadRead<_2D,uchar3> -> Crop(rects[n]) -> Resize<INTER_LINEAR, aspect>(dst_w x dst_h, background) ->
  * Mul<float3> -> Sub<float3> -> Div<float3> -> ColorConversion<COLOR_RGB2BGR> -> TensorWrite<float3>.
- * out: n planes of dst_h x dst_w packed float3.  n in {1,2,3,5,8,32,50}. */
+ * out: n planes of dst_h x dst_w packed float3.  Any n >= 1: the number of planes is a run-time value here (the reference
+ * fixes it with BATCH; its benchmarks/fusion/benchmark_horizontal_fusion.h:27-31 sweeps 1 .. 46 and names 120), up to 64
+ * planes per launch. */
 int fk_crop_resize_muls_bgr_tensor(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n,
                                    int dst_w, int dst_h, int aspect, const float background[3], const float mul[3],
                                    const float sub[3], const float div[3], float* out, void* stream);
@@ -56,13 +58,13 @@ int fk_single_op_f32c3(const void* src, int w, int h, size_t src_pitch, int is_a
 
 /* Horizontal fusion: PerThreadRead(array of n images) -> Crop(rects[n]) -> Resize<INTER_LINEAR>(dst) -> Div<float3> ->
  * Sub<float3> -> Div<float3> -> COLOR_RGB2BGR -> TensorSplit<float3> (memory_operations.h:195-226).
- * srcs: host array of n device pointers.  out: n x 3 x dst_h x dst_w planar float.  n in {1,2,3,5,8,32,50}. */
+ * srcs: host array of n device pointers.  out: n x 3 x dst_h x dst_w planar float.  Any n >= 1. */
 int fk_batch_crop_resize_norm_split(const void* const* srcs, int src_w, int src_h, size_t src_pitch, const fk_rect* rects,
                                     int n, int dst_w, int dst_h, const float div1[3], const float sub[3],
                                     const float div2[3], float* out, void* stream);
 
 /* Backwards vertical fusion: PerThreadRead<_2D,uchar3> -> Resize<INTER_LINEAR>(rs_w x rs_h) -> Crop(rects[n]) ->
- * Mul<float3> -> TensorWrite<float3>; no resized image is materialised.  out: n x tile_h x tile_w float3. */
+ * Mul<float3> -> TensorWrite<float3>; no resized image is materialised.  out: n x tile_h x tile_w float3.  Any n >= 1. */
 int fk_resize_crop_tiles(const void* src, int src_w, int src_h, size_t src_pitch, int rs_w, int rs_h, const fk_rect* rects,
                          int n, int tile_w, int tile_h, const float mul[3], float* out, void* stream);
 

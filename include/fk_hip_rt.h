@@ -30,9 +30,6 @@ enum { FKRT_H2D = 1, FKRT_D2H = 2, FKRT_D2D = 3, FKRT_H2H = 0 };
 int fkrt_device_count(int* count);
 int fkrt_set_device(int device);
 int fkrt_get_device(int* device);
-/* compute units of the current device (hipDeviceProp_t::multiProcessorCount; the reference reads the same property
- * where it sizes grids, core/execution_model/executors.h:262-287) */
-int fkrt_device_compute_units(int* count);
 
 int fkrt_stream_create(fkrt_stream* out);
 int fkrt_stream_destroy(fkrt_stream s);

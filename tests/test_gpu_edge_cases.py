@@ -167,8 +167,10 @@ def test_crop_at_the_last_row_and_column_of_the_buffer(fk, oracle):
 def test_argument_errors(fk, oracle):
     src = dev(oracle.bytes(1, (20, 30, 3)))
     out = torch.zeros((4, 8, 8, 3), device="cuda")
-    with pytest.raises(fk.FkError, match="unsupported"):
-        fk.crop_resize_muls_bgr_tensor(src, [(0, 0, 4, 4)] * 4, out, 0, (0,) * 3, (1,) * 3, (0,) * 3, (1,) * 3)
+    with pytest.raises(fk.FkError, match="unsupported"):  # an aspect-ratio mode that does not exist
+        fk.crop_resize_muls_bgr_tensor(src, [(0, 0, 4, 4)] * 4, out, 7, (0,) * 3, (1,) * 3, (0,) * 3, (1,) * 3)
+    with pytest.raises(fk.FkError, match="no planes"):
+        fk.crop_resize_muls_bgr_tensor(src, [], out[:0], 0, (0,) * 3, (1,) * 3, (0,) * 3, (1,) * 3)
     out = torch.zeros((1, 8, 8, 3), device="cuda")
     with pytest.raises(fk.FkError, match="outside"):
         fk.crop_resize_muls_bgr_tensor(src, [(25, 0, 10, 4)], out, 0, (0,) * 3, (1,) * 3, (0,) * 3, (1,) * 3)
