@@ -61,6 +61,11 @@ CAPI_SIGNATURES = {
     "fk_tensor_relayout_f32c3": [_i, _vp, _i, _i, _i, _vp, _vp],
     "fk_circular_tensor_read_f32c3": [_i, _i, _vp, _i, _i, _i, _vp, _vp],
     "fk_circular_tensor_update_u8c3_split_f32": [_vp, _i, _i, _sz, _f, _vp, _vp, _i, _i, _i, _vp],
+    "fk_conditional_copy_u8c3": [C.POINTER(C.c_void_p), _i, _i, _sz, _i, _i, C.POINTER(C.c_uint8), _vp, _vp],
+    "fk_conditional_resize_f32c3": [C.POINTER(C.c_void_p), _i, _i, _sz, _i, _i, _f3p, _i, _i, _vp, _vp],
+    "fk_muladd_midwrite_f32c3": [_vp, _i, _i, _sz, _f, _f, _vp, _sz, _vp, _sz, _vp],
+    "fk_batch_crop_cast_images": [_vp, _i, _i, _sz, _rp, _i, C.POINTER(C.c_void_p), _sz, _vp],
+    "fk_tensor_mul_f32c3": [_vp, _i, _i, _i, _f3p, _vp, _vp],
 }
 PACKED_TO_SPLIT, PACKED_TO_TRANSPOSED, SPLIT_TO_PACKED, TRANSPOSED_TO_PACKED = 0, 1, 2, 3
 ASCENDENT, DESCENDENT = 0, 1
@@ -417,3 +422,64 @@ def circular_tensor_update_u8c3_split_f32(frame, mul_v, tensor, ring, next_index
     _deferred = _call(capi.fk_circular_tensor_update_u8c3_split_f32, (p, w, h, pitch, float(mul_v), C.c_void_p(tensor.data_ptr()), C.c_void_p(ring.data_ptr()),
                                                                      batch, next_index, int(newest_first), _stream(stream)), defer)
     return _deferred if defer else (next_index + 1) % batch
+
+
+# ---- less common chain shapes: conditional batches, a write in the middle of a chain, a batch of output images, a tensor source ----
+def _same_images(srcs, dtype):
+    p0, w, h, pitch = _image(srcs[0], dtype)
+    for s in srcs:
+        assert _image(s, dtype)[1:] == (w, h, pitch)
+    return (C.c_void_p * len(srcs))(*[s.data_ptr() for s in srcs]), w, h, pitch
+
+
+def conditional_copy_u8c3(srcs, used, default, out, stream=None, defer=False):
+    """srcs: list of (H, W, 3) uint8 of one size/pitch; out: (n, H, W, 3) uint8 contiguous; planes from `used` on receive `default`."""
+    _, capi = load()
+    ptrs, w, h, pitch = _same_images(srcs, "uint8")
+    out = _dev(out, "uint8")
+    assert out.shape == (len(srcs), h, w, 3) and out.is_contiguous()
+    d = (C.c_uint8 * 3)(*[int(v) for v in default])
+    _deferred = _call(capi.fk_conditional_copy_u8c3, (ptrs, w, h, pitch, len(srcs), int(used), d, C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def conditional_resize_f32c3(srcs, used, default, out, stream=None, defer=False):
+    """srcs: list of (H, W, 3) uint8 of one size/pitch; out: (n, dst_h, dst_w, 3) float32 contiguous; planes from `used` on receive `default`."""
+    _, capi = load()
+    ptrs, w, h, pitch = _same_images(srcs, "uint8")
+    out = _dev(out, "float32")
+    assert out.shape[0] == len(srcs) and out.shape[3] == 3 and out.is_contiguous()
+    _deferred = _call(capi.fk_conditional_resize_f32c3, (ptrs, w, h, pitch, len(srcs), int(used), _f3(default), out.shape[2], out.shape[1],
+                                                           C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def muladd_midwrite_f32c3(src, mul_v, add_v, mid, out, stream=None, defer=False):
+    """src, mid, out: (H, W, 3) float32; mid receives src * mul_v, out receives src * mul_v + add_v."""
+    _, capi = load()
+    p, w, h, pitch = _image(src, "float32")
+    pm, wm, hm, pitch_m = _image(mid, "float32")
+    po, wo, ho, pitch_o = _image(out, "float32")
+    assert (w, h) == (wm, hm) == (wo, ho)
+    _deferred = _call(capi.fk_muladd_midwrite_f32c3, (p, w, h, pitch, mul_v, add_v, pm, pitch_m, po, pitch_o, _stream(stream)), defer)
+    return _deferred if defer else (mid, out)
+
+
+def batch_crop_cast_images(src, rects, outs, stream=None, defer=False):
+    """src: (H, W, 3) uint8; rects of one size; outs: list of (rh, rw, 3) float32 images of that size and one pitch."""
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    ptrs, ow, oh, out_pitch = _same_images(outs, "float32")
+    assert len(outs) == len(rects)
+    _deferred = _call(capi.fk_batch_crop_cast_images, (p, w, h, pitch, _rects(rects), len(rects), ptrs, out_pitch, _stream(stream)), defer)
+    return _deferred if defer else outs
+
+
+def tensor_mul_f32c3(src, mul, out, stream=None, defer=False):
+    """src, out: (planes, H, W, 3) float32 contiguous."""
+    _, capi = load()
+    src, out = _dev(src, "float32"), _dev(out, "float32")
+    assert src.shape == out.shape and src.shape[3] == 3 and src.is_contiguous() and out.is_contiguous()
+    planes, h, w, _ = src.shape
+    _deferred = _call(capi.fk_tensor_mul_f32c3, (C.c_void_p(src.data_ptr()), w, h, planes, _f3(mul), C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out

@@ -90,6 +90,36 @@ int fk_divergent4_u8c4(const void* src, int w, int h, size_t src_pitch, void* gr
 int fk_batch_crop_cast_tensor(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n,
                               int max_w, int max_h, float* out, void* stream);
 
+/* ---- less common chain shapes ---------------------------------------------------------------------------------- */
+
+/* executeOperations(std::array<Ptr2D<uchar3>, BATCH> input, activeBatch, defaultValue, Tensor<uchar3> output, stream)
+ * (fused_kernel.h:26-33 -> executors.h:77-84): PerThreadRead<_2D,uchar3>::build(used, def, images) ->
+ * PerThreadWrite<_3D,uchar3>, a batch read with PlanePolicy::CONDITIONAL_WITH_DEFAULT (batch_operations.h:218-241).
+ * srcs: host array of n device pointers to w x h images; planes z >= used receive `def` in every element.
+ * out: n planes of h x w packed uchar3.  1 <= n <= 64. */
+int fk_conditional_copy_u8c3(const void* const* srcs, int w, int h, size_t pitch, int n, int used, const uint8_t def[3], void* out,
+                             void* stream);
+/* PerThreadRead<_2D,uchar3>::build(images) -> Resize<INTER_LINEAR>::build(used, def, sizes) -> TensorWrite<float3>: the
+ * batch of resizes carries the policy and the fused batch keeps it (iop_fuser.h:57-62).  out: n planes of
+ * dst_h x dst_w packed float3; planes z >= used receive `def`.  1 <= n <= 64. */
+int fk_conditional_resize_f32c3(const void* const* srcs, int w, int h, size_t pitch, int n, int used, const float def[3], int dst_w,
+                                int dst_h, float* out, void* stream);
+/* PerThreadRead<_2D,float3> -> Mul<float3>(mul_v) -> PerThreadWrite<_2D,float3>(mid) -> Add<float3>(add_v) ->
+ * PerThreadWrite<_2D,float3>(out): a write in the middle of a chain stores the value and hands it on
+ * (fused_operation.h:49-62).  (The reference does this for a chain fused with .then(); given the same operations as
+ * separate arguments of executeOperations it ends the chain at the first write, data_parallel_patterns.h:77-79.  This
+ * library treats both forms alike.) */
+int fk_muladd_midwrite_f32c3(const void* src, int w, int h, size_t src_pitch, float mul_v, float add_v, void* mid, size_t mid_pitch,
+                             void* out, size_t out_pitch, void* stream);
+/* PerThreadRead<_2D,uchar3> -> Crop(rects[n]) -> Cast<uchar3,float3> -> PerThreadWrite<_2D,float3>::build(array of n
+ * images), a BatchWrite (batch_operations.h:43-75).  All rects have the size of the first; outs: host array of n device
+ * pointers to images of that size, rows out_pitch bytes apart.  1 <= n <= 64. */
+int fk_batch_crop_cast_images(const void* src, int w, int h, size_t pitch, const fk_rect* rects, int n, float* const* outs,
+                              size_t out_pitch, void* stream);
+/* TensorRead<float3> -> Mul<float3> -> TensorWrite<float3> (memory_operations.h:139-171, 173-193): planes x h x w packed
+ * float3 on both sides. */
+int fk_tensor_mul_f32c3(const void* src, int w, int h, int planes, const float mul[3], void* out, void* stream);
+
 /* ---- YUV front-end ------------------------------------------------------------------------------------------
  * A raw YUV image is ONE 2D allocation of base elements (uint8 for the 8-bit formats, uint16 with the sample in the
  * high bits for the 10-bit ones), rows src_pitch bytes apart, as RawImage<PF> describes it

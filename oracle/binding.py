@@ -88,12 +88,13 @@ def build(with_reference=True):
 class _Lib:
     """Thin numpy-facing wrapper; `ref=True` talks to the reference driver (literal host semantics)."""
 
-    def __init__(self, cdll, ref, yuv_cdll=None, bw_cdll=None, circ_cdll=None):
+    def __init__(self, cdll, ref, yuv_cdll=None, bw_cdll=None, circ_cdll=None, paths_cdll=None):
         self.c = cdll
         self.ref = ref
         self.yuv = yuv_cdll
         self.bw = bw_cdll
         self.circ = circ_cdll
+        self.paths = paths_cdll
         pre = "fkr_" if ref else "fko_"
         if circ_cdll is not None:
             _v = C.c_void_p
@@ -391,6 +392,61 @@ class _Lib:
         self._check(self.circ.fko_circular_tensor_update_u8c3_split_f32(_p(frame), w, h, frame.strides[0], float(mul_v), _p(tensor), _p(ring),
                                                                        tensor.shape[0], next_index, int(newest_first)))
 
+    # ---- conditional batches, a write in the middle of a chain, a batch of output images, a tensor as the source ----
+    def _paths_fn(self, name):
+        if self.paths is None:
+            raise RuntimeError("the checker library of the less common chain shapes is not built")
+        fn = getattr(self.paths, ("fkr_" if self.ref else "fko_") + name)
+        fn.restype = C.c_int
+        return fn
+
+    @staticmethod
+    def _pointers(arrays):
+        return (C.c_void_p * len(arrays))(*[a.ctypes.data for a in arrays])
+
+    def conditional_copy_u8c3(self, srcs, used, default):
+        """srcs: n images (h, w, 3) uint8 of one size -> (n, h, w, 3) uint8; planes from `used` on hold `default`."""
+        h, w, _ = srcs[0].shape
+        out = np.empty((len(srcs), h, w, 3), np.uint8)
+        d = np.asarray(default, np.uint8)
+        self._check(self._paths_fn("conditional_copy_u8c3")(self._pointers(srcs), _i(w), _i(h), _sz(srcs[0].strides[0]), _i(len(srcs)), _i(used),
+                                                             _p(d), _p(out)))
+        return out
+
+    def conditional_resize_f32c3(self, srcs, used, default, dst, quirk=0):
+        """srcs: n images (h, w, 3) uint8 of one size -> (n, dst_h, dst_w, 3) float32; planes from `used` on hold `default`."""
+        h, w, _ = srcs[0].shape
+        out = np.empty((len(srcs), dst[1], dst[0], 3), np.float32)
+        d = np.asarray(default, np.float32)
+        args = [self._pointers(srcs), _i(w), _i(h), _sz(srcs[0].strides[0]), _i(len(srcs)), _i(used), _p(d), _i(dst[0]), _i(dst[1])]
+        if not self.ref:
+            args.append(_i(quirk))
+        self._check(self._paths_fn("conditional_resize_f32c3")(*args, _p(out)))
+        return out
+
+    def muladd_midwrite_f32c3(self, src, mul_v, add_v):
+        """src: (h, w, 3) float32 -> (mid, out)."""
+        h, w, _ = src.shape
+        mid, out = np.empty_like(src), np.empty_like(src)
+        self._check(self._paths_fn("muladd_midwrite_f32c3")(_p(src), _i(w), _i(h), _sz(src.strides[0]), _f(mul_v), _f(add_v), _p(mid),
+                                                             _sz(mid.strides[0]), _p(out), _sz(out.strides[0])))
+        return mid, out
+
+    def batch_crop_cast_images(self, src, rects):
+        """src: (h, w, 3) uint8, rects of one size -> list of (rh, rw, 3) float32 images."""
+        h, w, _ = src.shape
+        outs = [np.empty((r[3], r[2], 3), np.float32) for r in rects]
+        self._check(self._paths_fn("batch_crop_cast_images")(_p(src), _i(w), _i(h), _sz(src.strides[0]), rect_array(rects), _i(len(rects)),
+                                                              self._pointers(outs), _sz(outs[0].strides[0])))
+        return outs
+
+    def tensor_mul_f32c3(self, src, mul):
+        """src: (planes, h, w, 3) float32 -> same shape."""
+        planes, h, w, _ = src.shape
+        out = np.empty_like(src)
+        self._check(self._paths_fn("tensor_mul_f32c3")(_p(src), _i(w), _i(h), _i(planes), _f3(mul), _p(out)))
+        return out
+
 
 _cache = {}
 
@@ -401,7 +457,7 @@ def oracle():
         if not os.path.exists(path):
             build(with_reference=False)
         cdll = C.CDLL(path)
-        _cache["o"] = _Lib(cdll, ref=False, yuv_cdll=cdll, bw_cdll=cdll, circ_cdll=cdll)
+        _cache["o"] = _Lib(cdll, ref=False, yuv_cdll=cdll, bw_cdll=cdll, circ_cdll=cdll, paths_cdll=cdll)
     return _cache["o"]
 
 
@@ -415,5 +471,7 @@ def reference():
         bw = C.CDLL(bw_path) if os.path.exists(bw_path) else None
         circ_path = os.path.join(_HERE, "_ref", "libfkref_circular.so")
         circ = C.CDLL(circ_path) if os.path.exists(circ_path) else None
-        _cache["r"] = _Lib(C.CDLL(path), ref=True, yuv_cdll=yuv, bw_cdll=bw, circ_cdll=circ) if os.path.exists(path) else None
+        paths_path = os.path.join(_HERE, "_ref", "libfkref_paths.so")
+        paths = C.CDLL(paths_path) if os.path.exists(paths_path) else None
+        _cache["r"] = _Lib(C.CDLL(path), ref=True, yuv_cdll=yuv, bw_cdll=bw, circ_cdll=circ, paths_cdll=paths) if os.path.exists(path) else None
     return _cache["r"]
