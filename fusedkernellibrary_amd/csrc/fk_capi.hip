@@ -185,6 +185,9 @@ int fk_crop_resize_muls_bgr_tensor(const void* src, int src_w, int src_h, size_t
                                    const float div[3], float* out, void* stream) {
     if (src == nullptr || out == nullptr || rects == nullptr || dst_w <= 0 || dst_h <= 0 || n <= 0) return bad_argument("null pointer, empty destination or no planes");
     if (!rects_inside(rects, n, src_w, src_h)) return bad_argument("crop rectangle outside the source image");
+    for (int i = 0; i < n; ++i) {
+        if (!interpolation_rows_exist(rects[i].y, rects[i].width, src_h)) return rows_missing();
+    }
     return guarded([&]() -> int {
         Stream s(stream);
         return readme_pipeline_any_ar(s, aspect, src, src_w, src_h, src_pitch, rects, n, dst_w, dst_h, background, mul, sub, div, out);
@@ -230,6 +233,9 @@ int fk_batch_crop_resize_norm_split(const void* const* srcs, int src_w, int src_
                                     void* stream) {
     if (srcs == nullptr || out == nullptr || rects == nullptr || dst_w <= 0 || dst_h <= 0 || n <= 0) return bad_argument("null pointer, empty destination or no planes");
     if (!rects_inside(rects, n, src_w, src_h)) return bad_argument("crop rectangle outside the source image");
+    for (int i = 0; i < n; ++i) {
+        if (!interpolation_rows_exist(rects[i].y, rects[i].width, src_h)) return rows_missing();
+    }
     return guarded([&]() -> int {
         Stream s(stream);
         split_pipeline(s, srcs, src_w, src_h, src_pitch, rects, n, dst_w, dst_h, div1, sub, div2, out);
@@ -241,6 +247,7 @@ int fk_resize_crop_tiles(const void* src, int src_w, int src_h, size_t src_pitch
                          int tile_w, int tile_h, const float mul[3], float* out, void* stream) {
     if (src == nullptr || out == nullptr || rects == nullptr || rs_w <= 0 || rs_h <= 0 || n <= 0) return bad_argument("null pointer, empty destination or no planes");
     if (!rects_inside(rects, n, rs_w, rs_h)) return bad_argument("tile outside the resized image");
+    if (!interpolation_rows_exist(0, src_w, src_h)) return rows_missing();
     for (int i = 0; i < n; ++i) {
         if (rects[i].width != tile_w || rects[i].height != tile_h) return bad_argument("every tile must be tile_w x tile_h");
     }
@@ -262,6 +269,7 @@ int fk_rgba2gray_u8c4(const void* src, int w, int h, size_t src_pitch, void* dst
 int fk_resize_mul_u8c4_f32c4(const void* src, int w, int h, size_t src_pitch, int dst_w, int dst_h, float mul_v, void* dst,
                              size_t dst_pitch, void* stream) {
     if (src == nullptr || dst == nullptr || w <= 0 || h <= 0 || dst_w <= 0 || dst_h <= 0) return bad_argument("null pointer or empty image");
+    if (!interpolation_rows_exist(0, w, h)) return rows_missing();
     return guarded([&]() -> int {
         Stream s(stream);
         run_sequence(s, resize_sequence(src, w, h, src_pitch, dst_w, dst_h, mul_v, dst, dst_pitch));
@@ -294,6 +302,7 @@ int fk_divergent4_u8c4(const void* src, int w, int h, size_t src_pitch, void* gr
         return bad_argument("null pointer or empty image");
     }
     if (!rects_inside(&rect_c, 1, w, h)) return bad_argument("crop rectangle outside the source image");
+    if (!interpolation_rows_exist(0, w, h)) return rows_missing();
     return guarded([&]() -> int {
         Stream s(stream);
         executeOperations<DivergentBatchTransformDPP<>>(

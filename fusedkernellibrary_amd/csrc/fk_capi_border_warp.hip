@@ -60,6 +60,7 @@ int fk_warp_u8c3_f32c3(int warp_type, const float* matrix, const void* src, int 
     if (src == nullptr || dst == nullptr || matrix == nullptr) return bad_argument("null pointer");
     if (w <= 0 || h <= 0 || dst_w <= 0 || dst_h <= 0) return bad_argument("empty image");
     if (src_pitch < static_cast<size_t>(w) * 3 || dst_pitch < static_cast<size_t>(dst_w) * 12) return bad_argument("pitch shorter than a row");
+    if (!interpolation_rows_exist(0, w, h)) return rows_missing();
     return guarded([&]() -> int {
         Stream s(stream);
         if (warp_type == FK_WARP_AFFINE) warp<WarpType::Affine>(s, matrix, src, w, h, src_pitch, dst_w, dst_h, dst, dst_pitch);

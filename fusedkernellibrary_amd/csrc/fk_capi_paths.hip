@@ -73,6 +73,7 @@ int fk_conditional_resize_f32c3(const void* const* srcs, int w, int h, size_t pi
                                 float* out, void* stream) {
     if (srcs == nullptr || out == nullptr || def == nullptr || w <= 0 || h <= 0 || dst_w <= 0 || dst_h <= 0) return bad_argument("null pointer or empty image");
     if (n <= 0 || n > MAX_PLANES) return bad_argument("a conditional batch takes 1 to 64 planes");
+    if (!interpolation_rows_exist(0, w, h)) return rows_missing();
     return guarded([&]() -> int {
         Stream s(stream);
         FK_FOR_CAPACITY(n, (conditional_resize<CAP>(s, srcs, w, h, pitch, n, used, def, dst_w, dst_h, out)))

@@ -138,6 +138,7 @@ int fk_yuv_crop_resize_norm_split(int format, int range, int primaries, const vo
     if (dst_w <= 0 || dst_h <= 0) return bad_argument("empty destination");
     if (crop.x < 0 || crop.y < 0 || crop.width <= 0 || crop.height <= 0 || crop.x + crop.width > width || crop.y + crop.height > height)
         return bad_argument("crop rectangle outside the source image");
+    if (!interpolation_rows_exist(crop.y, crop.width, height)) return rows_missing();
     return guarded([&]() -> int {
         Stream s(stream);
         int rc = FK_OK;

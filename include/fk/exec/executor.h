@@ -209,6 +209,20 @@ struct JobOf {
                     max_w = v.w > max_w ? v.w : max_w;
                     max_h = v.h > max_h ? v.h : max_h;
                 }
+                if constexpr (std::is_same_v<View, PlainView<Src>>) {
+                    // Windows of different sizes: every plane produces the extent of the largest, as the reference's
+                    // thread grid does (batch_operations.h:153-160: max width x max height for every plane); beside its
+                    // own window a plane then holds the parent image's pixels there (zero where the parent ends).
+                    bool ragged = false;
+                    for (size_t i = 0; i < used; ++i) ragged = ragged || job.plane[i].prog.view.w != max_w || job.plane[i].prog.view.h != max_h;
+                    if (ragged) {
+                        for (size_t i = 0; i < used; ++i) {
+                            job.plane[i].prog.view.w = max_w;
+                            job.plane[i].prog.view.h = max_h;
+                            job.plane[i].flags |= FLAG_WHOLE_BOX;
+                        }
+                    }
+                }
                 // thread columns per block: enough to span the widest row, at most the whole block
                 const unsigned groups = ceil_div(static_cast<unsigned>(max_w), Job::K);
                 unsigned shift = 0;

@@ -450,7 +450,7 @@ __device__ __attribute__((always_inline)) inline void fill_default(const Out& ou
 } // namespace dev
 
 // ---- pointwise ---------------------------------------------------------------------------------------------------
-enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u };
+enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_WHOLE_BOX = 8u };
 
 template <typename Prog, size_t N, typename Out, typename Defaults = NoDefaultPlanes>
 struct PointwiseJob {
@@ -585,19 +585,29 @@ struct PointwiseJob {
         const int x0 = (static_cast<int>(bx) * cols + (tid & (cols - 1))) * K;
         const int y = static_cast<int>(by) * (BLOCK_THREADS >> job.tx_shift) + (tid >> job.tx_shift);
 
+        // FLAG_WHOLE_BOX (a batch of windows of different sizes): every plane produces the extent of the largest, as the
+        // reference's thread grid does (batch_operations.h:153-160), so v.w x v.h is that box and elements beside the
+        // plane's own window are the parent image's pixels there; where the box leaves the parent image the source pixel
+        // is zero.
+        bool whole_box = false;
+        if constexpr (std::is_same_v<View, PlainView<Src>>) whole_box = (pl.flags & FLAG_WHOLE_BOX) != 0u;
         if constexpr (STAGE_IN || STAGE_OUT) {
             // block-uniform decisions
             const int bx0 = static_cast<int>(bx) * BLOCK_THREADS * K; // first pixel of the block
             const int span = v.w - bx0 < BLOCK_THREADS * K ? v.w - bx0 : BLOCK_THREADS * K;
-            if ((pl.flags & FLAG_VECTOR_IO) != 0u && job.tx_shift == 8u && y < v.h && span > 0 && span % K == 0) {
+            if ((pl.flags & FLAG_VECTOR_IO) != 0u && !whole_box && job.tx_shift == 8u && y < v.h && span > 0 && span % K == 0) {
                 if (span == BLOCK_THREADS * K) row_block<true>(job, pl, bx0, span, x0, y, bz, tid, lds);
                 else row_block<false>(job, pl, bx0, span, x0, y, bz, tid, lds);
                 return;
             }
         }
 
-        if (y >= v.h || x0 >= v.w) return; // also ends blocks that lie outside a smaller plane of a ragged batch
-        if ((pl.flags & FLAG_VECTOR_IO) != 0u && x0 + K <= v.w) {
+        if (y >= v.h || x0 >= v.w) return;
+        bool run_in_parent = true; // the thread's K pixels lie in the parent image
+        if constexpr (std::is_same_v<View, PlainView<Src>>) {
+            if (whole_box) run_in_parent = v.oy + y < v.img_h && v.ox + x0 + K <= v.img_w;
+        }
+        if ((pl.flags & FLAG_VECTOR_IO) != 0u && x0 + K <= v.w && run_in_parent) {
             Src in[K];
             Access::template load_group<K>(v, x0, y, in);
             OutPixel o[K];
@@ -607,8 +617,13 @@ struct PointwiseJob {
         } else {
             const int xe = x0 + K < v.w ? x0 + K : v.w;
             for (int x = x0; x < xe; ++x) {
-                const OutPixel o = dev::apply_tail(pl.prog.tail, Access::load_one(v, x, y));
-                dev::store_one(job.out, x, y, static_cast<int>(bz), o);
+                Src pixel{};
+                bool in_parent = true;
+                if constexpr (std::is_same_v<View, PlainView<Src>>) {
+                    if (whole_box) in_parent = v.oy + y < v.img_h && v.ox + x < v.img_w;
+                }
+                if (in_parent) pixel = Access::load_one(v, x, y);
+                dev::store_one(job.out, x, y, static_cast<int>(bz), dev::apply_tail(pl.prog.tail, pixel));
             }
         }
     }

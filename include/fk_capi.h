@@ -86,7 +86,10 @@ int fk_divergent4_u8c4(const void* src, int w, int h, size_t src_pitch, void* gr
                        void* stream);
 
 /* Ragged batch without resize: PerThreadRead -> Crop(rects[n]) -> Cast<uchar3,float3> -> TensorWrite<float3> into a
- * max_w x max_h x n tensor.  Elements outside a plane's own rect are left untouched. */
+ * max_w x max_h x n tensor.  Every plane receives the box of the largest width and the largest height among the rects,
+ * as the reference's thread grid covers it for every plane (batch_operations.h:153-160): beside its own rect a plane
+ * holds the source image's pixels there, and zero where the box leaves the source image (the reference reads past the
+ * image there).  Tensor elements outside that box are left untouched. */
 int fk_batch_crop_cast_tensor(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n,
                               int max_w, int max_h, float* out, void* stream);
 

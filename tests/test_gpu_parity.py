@@ -19,6 +19,14 @@ def dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
+def padded(a, extra):
+    """Copy `a` (h, w, c) into a device buffer whose rows are `extra` pixels longer: pitch != width * pixel size."""
+    h, w, c = a.shape
+    buf = torch.zeros((h, w + extra, c), dtype=torch.from_numpy(a).dtype, device="cuda")
+    buf[:, :w] = torch.from_numpy(a).cuda()
+    return buf[:, :w]
+
+
 def check(gpu, cpu):
     gpu = gpu.cpu().numpy()
     if gpu.dtype == np.float32 and not same_bits(gpu, cpu):
@@ -119,11 +127,29 @@ def test_divergent_one_launch(fk, oracle):
     check(bgr, oracle.rgba2bgr_sub_u8c4_f32c3(src, 0.5))
 
 
-def test_ragged_crops_leave_outside_untouched(fk, oracle):
+def test_ragged_crops_cover_the_largest_box_like_the_reference(fk, oracle):
+    """Crops of different sizes: every plane receives the box of the largest width and height, as the reference's thread
+    grid covers it (oracle with exec_all=1, pinned against the reference build); tensor elements beyond the box stay."""
     src = oracle.bytes(7, (120, 200, 3))
     rects = [(1, 2, 30, 20), (5, 5, 10, 25), (100, 60, 33, 7)]
-    want = oracle.batch_crop_cast_tensor(src, rects, (33, 25), exec_all=0, fill=-7.0)
-    out = torch.full((3, 25, 33, 3), -7.0, device="cuda")
+    want = np.full((3, 27, 36, 3), -7.0, np.float32)
+    want[:, :25, :33] = oracle.batch_crop_cast_tensor(src, rects, (33, 25), exec_all=1)
+    for extra in (0, 1, 3):  # tight and padded source rows: the wide and the element-wise paths
+        out = torch.full((3, 27, 36, 3), -7.0, device="cuda")
+        fk.batch_crop_cast_tensor(padded(src, extra) if extra else dev(src), rects, out)
+        torch.cuda.synchronize()
+        check(out, want)
+
+
+def test_ragged_crops_beyond_the_source_image_read_zero(fk, oracle):
+    """Where the largest box leaves the source image the reference reads past it; here the source pixel is zero."""
+    src = oracle.bytes(8, (40, 64, 3))
+    rects = [(0, 0, 50, 6), (60, 36, 4, 4), (20, 10, 8, 30)]  # the second plane's 50 x 30 box leaves the image on both sides
+    out = torch.full((3, 30, 50, 3), -7.0, device="cuda")
     fk.batch_crop_cast_tensor(dev(src), rects, out)
     torch.cuda.synchronize()
-    check(out, want)
+    got = out.cpu().numpy()
+    big = np.zeros((40 + 30, 64 + 50, 3), np.uint8)
+    big[:40, :64] = src
+    for z, (x, y, _, _) in enumerate(rects):
+        assert same_bits(got[z], big[y:y + 30, x:x + 50].astype(np.float32)), z
