@@ -41,6 +41,7 @@ _rp = C.POINTER(Rect)
 
 CAPI_SIGNATURES = {
     "fk_crop_resize_muls_bgr_tensor": [_vp, _i, _i, _sz, _rp, _i, _i, _i, _i, _f3p, _f3p, _f3p, _f3p, _vp, _vp],
+    "fk_crop_resize_muls_bgr_tensor_noalloc": [_vp, _i, _i, _sz, _rp, _i, _i, _i, _i, _f3p, _f3p, _f3p, _f3p, _vp, _vp],
     "fk_muladd_chain_f32c3": [_vp, _i, _i, _sz, _i, _f, _f, _vp, _sz, _vp],
     "fk_single_op_f32c3": [_vp, _i, _i, _sz, _i, _f, _vp, _sz, _vp],
     "fk_batch_crop_resize_norm_split": [C.POINTER(C.c_void_p), _i, _i, _sz, _rp, _i, _i, _i, _f3p, _f3p, _f3p, _vp, _vp],
@@ -185,6 +186,18 @@ def crop_resize_muls_bgr_tensor(src, rects, out, aspect, background, mul, sub, d
     assert n == len(rects) and out.is_contiguous()
     _deferred = _call(capi.fk_crop_resize_muls_bgr_tensor, (p, w, h, pitch, _rects(rects), n, dw, dh, aspect, _f3(background), _f3(mul),
                                                _f3(sub), _f3(div), C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def crop_resize_muls_bgr_tensor_noalloc(src, rects, out, aspect, background, mul, sub, div, stream=None, defer=False):
+    """The README pipeline through the entry point that allocates nothing (at most 64 planes); same arguments and results."""
+    _, capi = load()
+    p, w, h, pitch = _image(src, "uint8")
+    out = _dev(out, "float32")
+    n, dh, dw, _ = out.shape
+    assert n == len(rects) and out.is_contiguous()
+    _deferred = _call(capi.fk_crop_resize_muls_bgr_tensor_noalloc, (p, w, h, pitch, _rects(rects), n, dw, dh, aspect, _f3(background), _f3(mul),
+                                                                      _f3(sub), _f3(div), C.c_void_p(out.data_ptr()), _stream(stream)), defer)
     return _deferred if defer else out
 
 

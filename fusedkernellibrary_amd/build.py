@@ -45,7 +45,7 @@ def build_runtime():
     return out
 
 
-CAPI_SOURCES = ("fk_capi.hip", "fk_capi_yuv.hip", "fk_capi_border_warp.hip", "fk_capi_circular.hip", "fk_capi_paths.hip")
+CAPI_SOURCES = ("fk_capi.hip", "fk_capi_yuv.hip", "fk_capi_border_warp.hip", "fk_capi_circular.hip", "fk_capi_paths.hip", "fk_capi_noalloc.hip")
 
 
 def build_capi(extra_defines=(), name="libfk_capi.so"):

@@ -4,7 +4,7 @@
 #include <array>
 #include <vector>
 
-#include "fk_capi_common.h"
+#include "fk_capi_readme.h"
 
 using namespace fk;
 using namespace fk_capi;
@@ -17,16 +17,6 @@ std::string& last_error() {
 } // namespace fk_capi
 
 namespace {
-Rect rect_of(const fk_rect& r) { return Rect(static_cast<uint>(r.x), static_cast<uint>(r.y), r.width, r.height); }
-float3 f3(const float* v) { return float3{ v[0], v[1], v[2] }; }
-
-bool rects_inside(const fk_rect* r, int n, int w, int h) {
-    for (int i = 0; i < n; ++i) {
-        if (r[i].x < 0 || r[i].y < 0 || r[i].width <= 0 || r[i].height <= 0 || r[i].x + r[i].width > w || r[i].y + r[i].height > h) return false;
-    }
-    return true;
-}
-
 using Linear = InterpolationType;
 
 // A batch of n planes, n known at run time: the planes are built one by one with the same .then() chain (what the
@@ -50,23 +40,8 @@ void launch_planes(Stream& stream, const std::vector<PlaneIOp>& planes, const Re
 template <AspectRatio AR>
 void readme_pipeline(Stream& stream, const void* src, int w, int h, size_t pitch, const fk_rect* rects, int n, int dw, int dh,
                      const float* bg, const float* mul, const float* sub, const float* div, float* out) {
-    const auto read = PerThreadRead<ND::_2D, uchar3>::build(view2d<uchar3>(src, w, h, pitch));
-    const auto plane = [&](const fk_rect& r) {
-        const auto cropped = read.then(Crop<>::build(rect_of(r)));
-        const auto finish = [&](const auto& resized) {
-            return resized.then(Mul<float3>::build(f3(mul)))
-                .then(Sub<float3>::build(f3(sub)))
-                .then(Div<float3>::build(f3(div)))
-                .then(ColorConversion<ColorConversionCodes::COLOR_RGB2BGR, float3, float3>::build());
-        };
-        if constexpr (AR == AspectRatio::IGNORE_AR) {
-            return finish(cropped.then(Resize<Linear::INTER_LINEAR, AR>::build(Size(dw, dh))));
-        } else {
-            return finish(cropped.then(Resize<Linear::INTER_LINEAR, AR>::build(Size(dw, dh), f3(bg))));
-        }
-    };
-    std::vector<decltype(plane(rects[0]))> planes;
-    for (int i = 0; i < n; ++i) planes.push_back(plane(rects[i]));
+    std::vector<decltype(readme_plane<AR>(src, w, h, pitch, rects[0], dw, dh, bg, mul, sub, div))> planes;
+    for (int i = 0; i < n; ++i) planes.push_back(readme_plane<AR>(src, w, h, pitch, rects[i], dw, dh, bg, mul, sub, div));
     const size_t plane_floats = static_cast<size_t>(dw) * dh * 3;
     launch_planes(stream, planes, [&](size_t first, size_t count) {
         return TensorWrite<float3>::build(view3d<float3>(out + first * plane_floats, dw, dh, static_cast<int>(count), 1));
@@ -183,11 +158,7 @@ int fk_interpolate_y1_from_x(void) {
 int fk_crop_resize_muls_bgr_tensor(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n, int dst_w,
                                    int dst_h, int aspect, const float background[3], const float mul[3], const float sub[3],
                                    const float div[3], float* out, void* stream) {
-    if (src == nullptr || out == nullptr || rects == nullptr || dst_w <= 0 || dst_h <= 0 || n <= 0) return bad_argument("null pointer, empty destination or no planes");
-    if (!rects_inside(rects, n, src_w, src_h)) return bad_argument("crop rectangle outside the source image");
-    for (int i = 0; i < n; ++i) {
-        if (!interpolation_rows_exist(rects[i].y, rects[i].width, src_h)) return rows_missing();
-    }
+    if (const int rc = check_readme_arguments(src, src_w, src_h, rects, n, dst_w, dst_h, out)) return rc;
     return guarded([&]() -> int {
         Stream s(stream);
         return readme_pipeline_any_ar(s, aspect, src, src_w, src_h, src_pitch, rects, n, dst_w, dst_h, background, mul, sub, div, out);

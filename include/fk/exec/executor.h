@@ -301,6 +301,23 @@ inline void launch_job(const Job& job, unsigned planes, fkrt_stream stream) {
                 job, job.grid_x, job.grid_y, planes, job.lds_bytes(), stream);
 }
 
+// The same launch with the job read from `device_block`, device memory of `block_bytes` bytes that the caller brings (and
+// that no other launch in flight uses): one small kernel copies the job there from its kernel arguments, the chain's
+// kernel then reads it from there.  Nothing is allocated.  False when the job does not fit the block or the kernel
+// arguments.
+template <typename Job>
+inline bool launch_job_from(void* device_block, size_t block_bytes, const Job& job, unsigned planes, fkrt_stream stream) {
+    if (sizeof(Job) > block_bytes || sizeof(Job) > fkrt_max_kernarg_bytes()) return false;
+    if (job.grid_x == 0 || job.grid_y == 0 || planes == 0) return true; // nothing to do
+    Job* at = static_cast<Job*>(device_block);
+    void* store_argv[] = { const_cast<Job*>(&job), &at };
+    gpuErrchk(fkrt_launch(reinterpret_cast<const void*>(&store_job_kernel<Job>), 1, 1, 1, BLOCK_THREADS, 1, 1, store_argv, 0, stream));
+    void* argv[] = { &at };
+    gpuErrchk(fkrt_launch(reinterpret_cast<const void*>(&transform_kernel_indirect<Job>), job.grid_x, job.grid_y, planes, BLOCK_THREADS, 1, 1, argv,
+                          job.lds_bytes(), stream));
+    return true;
+}
+
 // (read, compute..., write) as (sender, receiver)
 template <typename Receiver>
 inline constexpr const Receiver& last_of(const Receiver& r) { return r; }
@@ -349,6 +366,16 @@ struct Executor<TransformDPP<ParArch::GPU_AMD, TFEN>> {
         using Plan = exec::JobOf<Sender, Receiver>;
         const auto job = Plan::make(seq.sender, seq.receiver);
         exec::launch_job(job, Plan::planes(seq.sender), stream.getHIPStream());
+    }
+    // The same with the chain's job kept in device memory that the caller brings instead of in the kernel arguments
+    // (this library's extension, for callers that must not allocate and hold such a block anyway; see
+    // exec::launch_job_from).  False when the job does not fit.
+    template <typename... IOps>
+    static inline bool executeOperationsFrom(void* device_block, size_t block_bytes, Stream_<ParArch::GPU_AMD>& stream, const IOps&... iOps) {
+        const auto seq = buildOperationSequence(iOps...);
+        using Plan = exec::JobOf<std::decay_t<decltype(seq.sender)>, std::decay_t<decltype(seq.receiver)>>;
+        const auto job = Plan::make(seq.sender, seq.receiver);
+        return exec::launch_job_from(device_block, block_bytes, job, Plan::planes(seq.sender), stream.getHIPStream());
     }
     // Convenience forms over buffers (executors.h:52-93).
     template <ND D, typename I, typename... IOps>

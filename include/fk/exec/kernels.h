@@ -1308,6 +1308,16 @@ __global__ __attribute__((amdgpu_flat_work_group_size(BLOCK_THREADS, BLOCK_THREA
              fk_dynamic_lds);
 }
 
+// Copies a job from the kernel-argument segment to device memory, for a launch that reads it from there (callers that
+// bring the memory for the job themselves).  One block.
+template <typename Job>
+__global__ __attribute__((amdgpu_flat_work_group_size(BLOCK_THREADS, BLOCK_THREADS))) void store_job_kernel(const Job job, Job* __restrict__ at) {
+    static_assert(sizeof(Job) % 4 == 0 && alignof(Job) >= 4, "a job is whole dwords");
+    const unsigned int* const from = reinterpret_cast<const unsigned int*>(&job_in_kernarg<Job>());
+    unsigned int* const to = reinterpret_cast<unsigned int*>(at);
+    for (unsigned i = static_cast<unsigned>(dev::thread_in_block()); i < sizeof(Job) / 4; i += BLOCK_THREADS) to[i] = from[i];
+}
+
 // Several different jobs in one launch ("divergent horizontal fusion"): the 1-D grid is cut into one contiguous
 // range of blocks per job, sized to that job alone, so that a small job does not pay for a large one's grid.
 template <typename... Jobs>

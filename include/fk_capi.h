@@ -46,6 +46,19 @@ int fk_crop_resize_muls_bgr_tensor(const void* src, int src_w, int src_h, size_t
                                    int dst_w, int dst_h, int aspect, const float background[3], const float mul[3],
                                    const float sub[3], const float div[3], float* out, void* stream);
 
+/* The same pipeline for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid it).  No counterpart in the reference, whose launches pass every parameter by value.  fk_crop_resize_muls_bgr_tensor
+ * keeps the chain's plane table in the kernel arguments or, above the runtime's limit for those, in a block that it
+ * allocates for the launch; this entry point keeps it in a fixed block of device memory that belongs to the library
+ * (FK_NOALLOC_MAX_JOB_BYTES per GPU, held until the process ends) and calls no allocating or freeing routine.  Same
+ * arguments and results; n <= FK_NOALLOC_MAX_PLANES, more returns FK_ERR_UNSUPPORTED.  All calls on one GPU share that
+ * block: calls that overlap there (other streams or host threads) race; calls in one stream do not. */
+#define FK_NOALLOC_MAX_PLANES 64
+#define FK_NOALLOC_MAX_JOB_BYTES 32768
+int fk_crop_resize_muls_bgr_tensor_noalloc(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n,
+                                           int dst_w, int dst_h, int aspect, const float background[3], const float mul[3],
+                                           const float sub[3], const float div[3], float* out, void* stream);
+
 /* Vertical fusion: PerThreadRead<_2D,float3> -> depth x alternating Mul<float3>(mul_v) / Add<float3>(add_v)
  * (operation 0 is Mul) -> PerThreadWrite<_2D,float3>, one launch.  depth in {1,2,4,8,16,32,64,128}.
  * (algorithms/basic_ops/arithmetic.h:22-88; benchmarks/numinstructions/benchmark_numinstructions_x_operation.h:68-99
