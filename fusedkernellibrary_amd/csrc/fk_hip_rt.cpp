@@ -3,6 +3,8 @@
 #include <hip/hip_runtime_api.h>
 
 #include <cstdlib>
+#include <cstring>
+#include <mutex>
 
 #include "fk_hip_rt.h"
 
@@ -66,16 +68,62 @@ int fkrt_launch(const void* kernel, unsigned grid_x, unsigned grid_y, unsigned g
     return static_cast<int>(hipGetLastError());
 }
 
+// Staged parameter blocks leave the host through a small ring of pinned buffers that this layer owns: the caller's block
+// is copied into a ring slot on the spot (so it may go out of scope at once), and the copy to the device is a true
+// asynchronous copy from pinned memory, ordered in the stream like the kernel that reads it.  A slot is taken again only
+// after the event recorded behind its copy has completed.
+namespace {
+struct StagingRing {
+    static constexpr int SLOTS = 8;
+    static constexpr size_t MIN_BYTES = 64 * 1024;
+    std::mutex lock;
+    void* host[SLOTS] = {};
+    size_t bytes[SLOTS] = {};
+    hipEvent_t copied[SLOTS] = {};
+    bool in_flight[SLOTS] = {};
+    int next = 0;
+};
+StagingRing& staging_ring() {
+    static StagingRing ring; // lives until the process ends; its pinned buffers are released with the process
+    return ring;
+}
+} // namespace
+
 int fkrt_params_upload(void** device_out, const void* host_src, size_t bytes, fkrt_stream s) {
+    StagingRing& ring = staging_ring();
+    std::lock_guard<std::mutex> hold(ring.lock);
+    const int slot = ring.next;
+    ring.next = (ring.next + 1) % StagingRing::SLOTS;
+    hipError_t e = hipSuccess;
+    if (ring.copied[slot] == nullptr) {
+        e = hipEventCreateWithFlags(&ring.copied[slot], hipEventDisableTiming);
+        if (e != hipSuccess) return static_cast<int>(e);
+    }
+    if (ring.in_flight[slot]) { // the copy that last used this slot must have left it
+        e = hipEventSynchronize(ring.copied[slot]);
+        if (e != hipSuccess) return static_cast<int>(e);
+        ring.in_flight[slot] = false;
+    }
+    if (ring.bytes[slot] < bytes) {
+        if (ring.host[slot] != nullptr) (void)hipHostFree(ring.host[slot]);
+        ring.host[slot] = nullptr;
+        ring.bytes[slot] = 0;
+        const size_t wanted = bytes > StagingRing::MIN_BYTES ? bytes : StagingRing::MIN_BYTES;
+        e = hipHostMalloc(&ring.host[slot], wanted, hipHostMallocPortable);
+        if (e != hipSuccess) return static_cast<int>(e);
+        ring.bytes[slot] = wanted;
+    }
+    std::memcpy(ring.host[slot], host_src, bytes);
     void* d = nullptr;
-    hipError_t e = hipMallocAsync(&d, bytes, as_stream(s));
+    e = hipMallocAsync(&d, bytes, as_stream(s));
     if (e != hipSuccess) return static_cast<int>(e);
-    // pageable source: the runtime stages it before returning, so the caller's block may go out of scope
-    e = hipMemcpyAsync(d, host_src, bytes, hipMemcpyHostToDevice, as_stream(s));
+    e = hipMemcpyAsync(d, ring.host[slot], bytes, hipMemcpyHostToDevice, as_stream(s));
+    if (e == hipSuccess) e = hipEventRecord(ring.copied[slot], as_stream(s));
     if (e != hipSuccess) {
         (void)hipFreeAsync(d, as_stream(s));
         return static_cast<int>(e);
     }
+    ring.in_flight[slot] = true;
     *device_out = d;
     return 0;
 }

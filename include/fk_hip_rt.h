@@ -54,7 +54,8 @@ int fkrt_launch(const void* kernel, unsigned grid_x, unsigned grid_y, unsigned g
 
 /* Stream-ordered staging of a parameter block that is too large for the kernel-argument segment: copies `bytes`
  * from host memory into a device buffer that stays valid for work already enqueued on `s`; release with
- * fkrt_params_release after enqueueing the kernel that reads it. */
+ * fkrt_params_release after enqueueing the kernel that reads it.  `host_src` is copied before the call returns (into
+ * a pinned buffer of a small ring that this layer owns) and may be released at once. */
 int fkrt_params_upload(void** device_out, const void* host_src, size_t bytes, fkrt_stream s);
 int fkrt_params_release(void* device_params, fkrt_stream s);
 
