@@ -636,8 +636,8 @@ constexpr int RESIZE_TILE_W = 64;
 constexpr int RESIZE_GROUP_ROWS = 4;      // rows that a wave finishes, and writes, at a time
 constexpr int RESIZE_MAX_WAVE_ROWS = 16;
 constexpr int RESIZE_LDS_DWORDS = 6144;   // source tile capacity (24 KiB)
-// A taller tile is chosen only while the grid keeps this many blocks (measured: 50 planes of 224 x 224 are faster as 1400
-// tiles of 64 x 32 than as 2800 of 64 x 16, five planes of 1920 x 1080 slower as 2550 tiles of 64 x 64 than as 5100 of 64 x 32).
+// A taller tile is chosen only while the grid keeps this many blocks (measured: five planes of 1920 x 1080 are slower as
+// 2550 tiles of 64 x 64 than as 5100 of 64 x 32), and only when every plane's tiles are staged in LDS.
 constexpr size_t RESIZE_MIN_BLOCKS_16 = 4096, RESIZE_MIN_BLOCKS_8 = 1024;
 static_assert(RESIZE_TILE_W == 64, "a lane per column");
 
@@ -761,17 +761,18 @@ struct ResizeJob {
     // Chooses the tile height and the LDS size from the factors of the first `count` planes; grid_x has been decided,
     // max_h is the tallest plane.  Returns the number of tile rows (grid_y).
     unsigned plan(size_t count, int max_h, unsigned forced_wave_rows) {
-        // the tallest tile that still leaves the grid enough blocks, and whose source boxes fit the LDS wherever those of
-        // the smallest tile do
+        // the tallest tile that still leaves the grid enough blocks, and whose source boxes all fit the LDS
         const auto blocks = [&](unsigned wr) { return count * grid_x * ((static_cast<unsigned>(max_h) + 4u * wr - 1u) / (4u * wr)); };
         const auto staged_planes = [&](unsigned wr) {
             unsigned n = 0;
             for (size_t i = 0; i < count; ++i) n += staged_tile_dwords(plane[i].view.fx, plane[i].view.fy, 4 * static_cast<int>(wr)) != 0u ? 1u : 0u;
             return n;
         };
+        // (tiles whose taps come straight from memory stay small: measured, eight 1920x1080 planes to 1280x720 take 30.8 us
+        // as 64 x 16 tiles and 33.8 us as 64 x 32, although the taller tile executes fewer instructions)
         wave_rows = RESIZE_GROUP_ROWS;
-        if (blocks(16) >= RESIZE_MIN_BLOCKS_16 && staged_planes(16) == staged_planes(RESIZE_GROUP_ROWS)) wave_rows = 16;
-        else if (blocks(8) >= RESIZE_MIN_BLOCKS_8 && staged_planes(8) == staged_planes(RESIZE_GROUP_ROWS)) wave_rows = 8;
+        if (blocks(16) >= RESIZE_MIN_BLOCKS_16 && staged_planes(16) == count) wave_rows = 16;
+        else if (blocks(8) >= RESIZE_MIN_BLOCKS_8 && staged_planes(8) == count) wave_rows = 8;
         if (forced_wave_rows == 4u || forced_wave_rows == 8u || forced_wave_rows == 16u) wave_rows = forced_wave_rows;
         tile_dwords = 0;
         for (size_t i = 0; i < count; ++i) {
@@ -1151,6 +1152,27 @@ struct ResizeJob {
 // gather in flight per wave; with K = 4 a thread issues the reads of four elements before it uses any of them, provided
 // the chain's read is straight-line code (lanes past the end of a row read its last element again instead of branching
 // around the read).  K = 1 is kept for small outputs, which need every wave they can get.
+namespace dev {
+// Blocks are handed to the eight XCDs in turn, in launch order, and each XCD has its own L2.  Neighbouring tiles read
+// source lines in common (the rows and columns where their boxes meet, every line of a slanted row for a warp): with
+// the blocks as they come, nearly every such line is fetched by several XCDs.  Here the block with launch number l works
+// on tile (l % 8) * total / 8 + l / 8 instead: each XCD covers one contiguous band of the output, and a source line is
+// fetched by the one or two XCDs whose bands need it.  For launches whose tiles all cost the same: a band of cheap tiles
+// (the planes of a batch that only receive a default value, the bars beside a resized image) would leave its XCD idle
+// early; measured on the resize kernel, eight 1920x1080 planes of which five are resized: 31.2 -> 40.8 us.
+__device__ __attribute__((always_inline)) inline void xcd_band_block(unsigned& bx, unsigned& by, unsigned& bz, const unsigned gx, const unsigned gy,
+                                                                    const unsigned gz) {
+    const unsigned total = gx * gy * gz;
+    const unsigned l = bx + gx * (by + gy * bz);
+    const unsigned share = total >> 3, rest = total & 7u, xcd = l & 7u; // the first `rest` XCDs take one block more
+    const unsigned tile = xcd * share + (xcd < rest ? xcd : rest) + (l >> 3);
+    const unsigned row = tile / gx;
+    bx = tile - row * gx;
+    bz = row / gy;
+    by = row - bz * gy;
+}
+} // namespace dev
+
 constexpr unsigned GENERIC_WIDE_MIN_ELEMS = 1u << 22;
 template <typename Sender, typename Receiver>
 struct GenericJob {
@@ -1161,6 +1183,7 @@ struct GenericJob {
     ActiveThreads active;
     unsigned grid_x, grid_y;
     unsigned wide; // 4 elements per thread instead of 1
+    unsigned xcd_bands; // tiles dealt out in one band per XCD (dev::xcd_band_block)
     // A packed receiver whose pixels are not whole dwords (three bytes, say) would be written with byte stores.  With
     // four elements per thread such a job gives a thread four neighbouring pixels instead of four that are 64 apart:
     // they are sizeof(pixel) whole dwords of the row, packed in registers and stored at once.  (For every other job
@@ -1269,6 +1292,7 @@ struct GenericJob {
         }
     }
     __device__ __attribute__((always_inline)) static inline void run(const GenericJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char*) {
+        if (job.xcd_bands != 0u) dev::xcd_band_block(bx, by, bz, job.grid_x, job.grid_y, job.active.z);
         if constexpr (PACKS_ROWS) { // the only jobs that are compiled with the neighbour form
             if (job.wide != 0u && job.packs_rows != 0u) {
                 body<4, true>(job, bx, by, bz);
