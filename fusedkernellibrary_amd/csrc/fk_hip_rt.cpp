@@ -68,23 +68,28 @@ int fkrt_launch(const void* kernel, unsigned grid_x, unsigned grid_y, unsigned g
     return static_cast<int>(hipGetLastError());
 }
 
-// Staged parameter blocks leave the host through a small ring of pinned buffers that this layer owns: the caller's block
-// is copied into a ring slot on the spot (so it may go out of scope at once), and the copy to the device is a true
-// asynchronous copy from pinned memory, ordered in the stream like the kernel that reads it.  A slot is taken again only
-// after the event recorded behind its copy has completed.
+// Staged parameter blocks go through a small ring of slots that this layer owns, each a pinned host buffer and a device
+// buffer of the same size (64 KiB, grown when a larger block comes).  The caller's block is copied into the slot's host
+// buffer on the spot (so it may go out of scope at once), and from there to the slot's device buffer with a true
+// asynchronous copy from pinned memory, ordered in the stream like the kernel that reads it.  fkrt_params_release, which
+// the caller issues after enqueueing that kernel, records the slot's event behind it; a slot is taken again only after
+// that event has completed.  Nothing is allocated per launch (a stream-ordered allocation and its release cost more
+// than the copy).  Slots belong to the device that was current when their buffers were made.
 namespace {
 struct StagingRing {
     static constexpr int SLOTS = 8;
     static constexpr size_t MIN_BYTES = 64 * 1024;
     std::mutex lock;
     void* host[SLOTS] = {};
+    void* device[SLOTS] = {};
     size_t bytes[SLOTS] = {};
-    hipEvent_t copied[SLOTS] = {};
+    int owner[SLOTS] = {}; // device of the slot's buffers
+    hipEvent_t done[SLOTS] = {};
     bool in_flight[SLOTS] = {};
     int next = 0;
 };
 StagingRing& staging_ring() {
-    static StagingRing ring; // lives until the process ends; its pinned buffers are released with the process
+    static StagingRing ring; // lives until the process ends; its buffers are released with the process
     return ring;
 }
 } // namespace
@@ -94,41 +99,48 @@ int fkrt_params_upload(void** device_out, const void* host_src, size_t bytes, fk
     std::lock_guard<std::mutex> hold(ring.lock);
     const int slot = ring.next;
     ring.next = (ring.next + 1) % StagingRing::SLOTS;
-    hipError_t e = hipSuccess;
-    if (ring.copied[slot] == nullptr) {
-        e = hipEventCreateWithFlags(&ring.copied[slot], hipEventDisableTiming);
-        if (e != hipSuccess) return static_cast<int>(e);
-    }
-    if (ring.in_flight[slot]) { // the copy that last used this slot must have left it
-        e = hipEventSynchronize(ring.copied[slot]);
+    int current = 0;
+    hipError_t e = hipGetDevice(&current);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (ring.in_flight[slot]) { // the kernel that last read this slot must have finished
+        e = hipEventSynchronize(ring.done[slot]);
         if (e != hipSuccess) return static_cast<int>(e);
         ring.in_flight[slot] = false;
     }
-    if (ring.bytes[slot] < bytes) {
+    if (ring.bytes[slot] < bytes || ring.owner[slot] != current || ring.done[slot] == nullptr) {
         if (ring.host[slot] != nullptr) (void)hipHostFree(ring.host[slot]);
-        ring.host[slot] = nullptr;
+        if (ring.device[slot] != nullptr) (void)hipFree(ring.device[slot]);
+        if (ring.done[slot] != nullptr) (void)hipEventDestroy(ring.done[slot]);
+        ring.host[slot] = ring.device[slot] = nullptr;
+        ring.done[slot] = nullptr;
         ring.bytes[slot] = 0;
         const size_t wanted = bytes > StagingRing::MIN_BYTES ? bytes : StagingRing::MIN_BYTES;
         e = hipHostMalloc(&ring.host[slot], wanted, hipHostMallocPortable);
+        if (e == hipSuccess) e = hipMalloc(&ring.device[slot], wanted);
+        if (e == hipSuccess) e = hipEventCreateWithFlags(&ring.done[slot], hipEventDisableTiming);
         if (e != hipSuccess) return static_cast<int>(e);
         ring.bytes[slot] = wanted;
+        ring.owner[slot] = current;
     }
     std::memcpy(ring.host[slot], host_src, bytes);
-    void* d = nullptr;
-    e = hipMallocAsync(&d, bytes, as_stream(s));
+    e = hipMemcpyAsync(ring.device[slot], ring.host[slot], bytes, hipMemcpyHostToDevice, as_stream(s));
     if (e != hipSuccess) return static_cast<int>(e);
-    e = hipMemcpyAsync(d, ring.host[slot], bytes, hipMemcpyHostToDevice, as_stream(s));
-    if (e == hipSuccess) e = hipEventRecord(ring.copied[slot], as_stream(s));
-    if (e != hipSuccess) {
-        (void)hipFreeAsync(d, as_stream(s));
-        return static_cast<int>(e);
-    }
+    // (should the caller never release it, the slot still waits for this copy before it is used again)
+    e = hipEventRecord(ring.done[slot], as_stream(s));
+    if (e != hipSuccess) return static_cast<int>(e);
     ring.in_flight[slot] = true;
-    *device_out = d;
+    *device_out = ring.device[slot];
     return 0;
 }
 int fkrt_params_release(void* device_params, fkrt_stream s) {
-    return static_cast<int>(hipFreeAsync(device_params, as_stream(s)));
+    StagingRing& ring = staging_ring();
+    std::lock_guard<std::mutex> hold(ring.lock);
+    for (int slot = 0; slot < StagingRing::SLOTS; ++slot) {
+        if (ring.device[slot] == device_params && device_params != nullptr) {
+            return static_cast<int>(hipEventRecord(ring.done[slot], as_stream(s))); // behind the kernel that reads the slot
+        }
+    }
+    return static_cast<int>(hipErrorInvalidValue);
 }
 
 size_t fkrt_max_kernarg_bytes(void) {
@@ -139,7 +151,7 @@ size_t fkrt_max_kernarg_bytes(void) {
             if (v >= 256) return static_cast<size_t>(v);
         }
         // Arguments of up to 64 KiB were verified to arrive intact on ROCm 7.2 / gfx950, also with thousands of launches
-        // in flight on two streams; half of that is used.  The staged block costs a launch 6-13 us.
+        // in flight on two streams; half of that is used.
         return static_cast<size_t>(32768);
     }();
     return limit;

@@ -53,9 +53,11 @@ int fkrt_launch(const void* kernel, unsigned grid_x, unsigned grid_y, unsigned g
                 unsigned block_y, unsigned block_z, void** args, size_t lds_bytes, fkrt_stream s);
 
 /* Stream-ordered staging of a parameter block that is too large for the kernel-argument segment: copies `bytes`
- * from host memory into a device buffer that stays valid for work already enqueued on `s`; release with
- * fkrt_params_release after enqueueing the kernel that reads it.  `host_src` is copied before the call returns (into
- * a pinned buffer of a small ring that this layer owns) and may be released at once. */
+ * from host memory into a device buffer that stays valid until the work enqueued on `s` up to the matching
+ * fkrt_params_release has run; call that after enqueueing the kernel that reads the block.  `host_src` is copied before
+ * the call returns and may be released at once.  The buffers come from a ring of eight slots that this layer owns (a
+ * pinned host buffer and a device buffer each): nothing is allocated per call, and a ninth upload waits on the host
+ * until the first slot's kernel has finished. */
 int fkrt_params_upload(void** device_out, const void* host_src, size_t bytes, fkrt_stream s);
 int fkrt_params_release(void* device_params, fkrt_stream s);
 
