@@ -57,7 +57,8 @@ int fkrt_launch(const void* kernel, unsigned grid_x, unsigned grid_y, unsigned g
  * fkrt_params_release has run; call that after enqueueing the kernel that reads the block.  `host_src` is copied before
  * the call returns and may be released at once.  The buffers come from a ring of eight slots that this layer owns (a
  * pinned host buffer and a device buffer each): nothing is allocated per call, and a ninth upload waits on the host
- * until the first slot's kernel has finished. */
+ * until the first slot's kernel has finished.  At most eight blocks may be between their upload and their release at
+ * any time (host threads that stage blocks concurrently: at most eight of them). */
 int fkrt_params_upload(void** device_out, const void* host_src, size_t bytes, fkrt_stream s);
 int fkrt_params_release(void* device_params, fkrt_stream s);
 
