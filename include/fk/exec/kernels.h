@@ -1066,6 +1066,28 @@ struct ResizeJob {
                         }
                     }
                 }
+            } else if constexpr (RAW_SOURCE) {
+                // Taps straight from memory, from a box of moderate size (down-scaling by up to about 1.7): every line of the
+                // box is touched once, now, with one load per 128-byte line whose value is not used, so that the gathers,
+                // which come after the lanes' set-up and wait for sixteen taps at a time, find the lines on their way
+                // (measured: eight 1920x1080 planes to 1280x720 31.3 -> 28.6 us; for larger boxes the touches cost more than
+                // they bring, 3x down-scaling 6.3 -> 7.6 us).
+                const int last_byte = s.w * static_cast<int>(sizeof(Src)) - 4; // last dword that lies wholly inside a window row
+                if (rows * cols <= 3 * tile_px + 256 && last_byte >= 0) {
+                    const int row_bytes = cols * static_cast<int>(sizeof(Src));
+                    const int first_byte = sx_lo * static_cast<int>(sizeof(Src));
+                    const int lines = (row_bytes + 127) / 128 + 1;
+                    const int total = rows * lines;
+                    for (int i = tid; i < total; i += BLOCK_THREADS) {
+                        const int r = i / lines, l = i - r * lines;
+                        const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
+                        int at = first_byte + l * 128;
+                        at = at < last_byte ? at : last_byte;
+                        at = at < 0 ? 0 : at;
+                        const unsigned int touched = dev::load_dword_from_row(window, static_cast<unsigned>(sy) * s.pitch + static_cast<unsigned>(at) + 1u);
+                        asm volatile("" ::"v"(touched));
+                    }
+                }
             }
         }
         dev::block_sync();
