@@ -69,10 +69,11 @@ def build_capi(extra_defines=(), name="libfk_capi.so"):
 
 
 def build_cpp_tests():
-    """The C++ programs under tests/cpp: the host-side API conformance check and the README example as user code."""
+    """The C++ programs under tests/cpp: the host-side API conformance check, the README example and the executor surface as
+    user code, and a translation unit that includes the HIP runtime's own header before the library's."""
     tests = os.path.join(ROOT, "tests", "cpp")
     outs = []
-    for name in ("conformance", "readme_dropin", "api_gpu"):
+    for name in ("conformance", "readme_dropin", "api_gpu", "hip_header_coexistence"):
         out = os.path.join(tests, name)
         _run([hipcc(), "-x", "hip", os.path.join(tests, name + ".cpp"), "-I" + INCLUDE, *DEVICE_FLAGS, "-L" + HERE, "-lfk_hip_rt",
               "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/../../fusedkernellibrary_amd", "-o", out])

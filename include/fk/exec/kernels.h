@@ -4,13 +4,14 @@
 //   PointwiseJob  element-wise chains over a PlainView or a YuvView: each thread owns K consecutive pixels of a row so
 //                 that both the source and the destination bytes of a thread are whole 16-byte (or 8/4-byte)
 //                 transactions (a YUV thread loads its luma run and the chroma pairs that cover it);
-//   ResizeJob     bilinear resize (with optional inner/outer crop and aspect-ratio border): a block owns a 64x16 output
-//                 tile, four pixels per thread; it stages the source bounding box of the tile in LDS, one dword-aligned
-//                 slot per source pixel (after the operations fused before the resize, e.g. YUV -> RGB, so those run
-//                 once per source pixel), and takes the 2x2 taps from there; tiles that gain nothing from it (strong
-//                 down-scaling, no tap reuse) read their taps straight from memory; packed outputs leave through LDS
-//                 as whole 16-byte pieces;
-//   GenericJob    one thread per output element through Operation::exec, for any chain the views cannot describe.
+//   ResizeJob     bilinear resize (with optional inner/outer crop and aspect-ratio border): a block owns an output tile
+//                 of 64 columns by 16, 32 or 64 rows, a wave a quarter of its rows, a lane one column of them; the block
+//                 stages the source bounding box of the tile in LDS as float taps (after the operations fused before the
+//                 resize, e.g. YUV -> RGB, so those and the conversion run once per source pixel) and takes the 2x2 taps
+//                 from there; tiles that gain nothing from it (down-scaling, no tap reuse) read their taps straight
+//                 from memory; outputs are stored from registers, a row of 64 neighbouring pixels per wave;
+//   GenericJob    one thread per output element (or four) through Operation::exec, for any chain the views cannot
+//                 describe.
 // blockIdx.z selects the plane of a batch; blocks that start outside their plane's own extent return at once.
 // What one thread computes per element is the reference's TransformDPP::exec -> read -> compute... -> write
 // (core/execution_model/data_parallel_patterns.h:120-181,254-268); the traversal, vector widths and LDS staging
@@ -21,12 +22,15 @@
 #include "fk/exec/views.h"
 
 // clang emits a host-side stub for every __global__ function that refers to this runtime entry point; kernels are
-// launched through fkrt_launch (which calls it with the stub's address), so only the declaration is needed here.
+// launched through fkrt_launch (which calls it with the stub's address), so only the declaration is needed here.  A
+// translation unit that has included the HIP runtime's own header before this one already has it.
+#if !defined(HIP_INCLUDE_HIP_HIP_RUNTIME_API_H)
 struct fk_launch_dim3 {
     unsigned x, y, z;
 };
 extern "C" int hipLaunchKernel(const void* function_address, fk_launch_dim3 grid, fk_launch_dim3 block, void** args,
                                size_t lds_bytes, struct ihipStream_t* stream);
+#endif
 
 namespace fk {
 namespace exec {

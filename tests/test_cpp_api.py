@@ -43,6 +43,16 @@ def test_executor_surface_as_user_code():
 
 
 @pytest.mark.gpu
+def test_user_code_that_includes_the_hip_runtime_header_first():
+    """<hip/hip_runtime.h> before <fused_kernel/fused_kernel.h> in one translation unit: a chain on a stream made by the
+    HIP API, timed with HIP events."""
+    exe = os.path.join(HERE, "cpp", "hip_header_coexistence")
+    assert os.path.exists(exe), "tests/cpp/hip_header_coexistence is not built"
+    proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=100)
+    assert proc.returncode == 0 and "hip_header_coexistence ok" in proc.stdout, proc.stdout
+
+
+@pytest.mark.gpu
 def test_reference_benchmark_sweeps_run_and_check_themselves():
     """The reference's four benchmark sweeps as user code (two timed iterations here): every sweep point compares its two
     variants with each other and with the closed-form result, and the program exits non-zero on any mismatch."""
