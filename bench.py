@@ -178,7 +178,7 @@ def build_workloads(fk, oracle, pool, only=None):
     def add(*a, **k):
         made.append(Workload(*a, **k))
 
-    # ---- C1: the README pipeline (BASELINE configuration 1's chain) --------------------------------------------------
+    # ---- C1: the README pipeline (the reference's README example) --------------------------------------------------
     def readme(name, rects, dst, note):
         if not want(name):
             return
@@ -196,13 +196,13 @@ def build_workloads(fk, oracle, pool, only=None):
         add(name, lambda i: calls[i % k](), n * dst[0] * dst[1], alg, "transform_kernel<ResizeJob<uchar3 -> float3, README tail, N = 5>>", k, verify, note)
 
     readme("C1_readme_60x60x5", [(0, 0, 34, 25), (10, 10, 70, 15), (20, 20, 60, 59), (30, 30, 20, 23), (40, 40, 12, 11)], (60, 60),
-           "BASELINE configuration 1 at its literal shape: 234 KB moved, bound by launch latency")
+           "benchmark configuration 1 at its literal shape: 234 KB moved, bound by launch latency")
     readme(HEADLINE, [(64 * i, 48 * i, 1024, 768) for i in range(5)], (1920, 1080),
            "4:3 crops into a 16:9 target under PRESERVE_AR: a quarter of the output is the bars beside the image")
     readme("C1_nobars_5x1024x576_to_1920x1080", [(64 * i, 48 * i, 1024, 576) for i in range(5)], (1920, 1080),
            "16:9 crops: every output pixel is resampled")
 
-    # ---- C2: vertical fusion, depth 16 (BASELINE configuration 2) ----------------------------------------------------
+    # ---- C2: vertical fusion, depth 16 (benchmark configuration 2) ----------------------------------------------------
     name = f"C2_vertical_fusion_depth{DEPTH}"
     if want(name):
         alg2 = 2 * N4K * 12
@@ -217,7 +217,7 @@ def build_workloads(fk, oracle, pool, only=None):
         add(name, lambda i: calls2[i % k2](), N4K, alg2, f"transform_kernel<PointwiseJob<float3 -> float3, depth {DEPTH}>>", k2, verify_c2,
             "3840x2160 float3, PerThreadRead -> 16 alternating Mul/Add -> PerThreadWrite in one launch")
 
-    # ---- C3: 50 crops of 50 images -> 224x224x3x50 planar (BASELINE configuration 3) ---------------------------------
+    # ---- C3: 50 crops of 50 images -> 224x224x3x50 planar (benchmark configuration 3) ---------------------------------
     if want("C3_batch50_224x224_split"):
         n, w, h = 50, 1920, 1080
         rects3 = []
@@ -239,7 +239,7 @@ def build_workloads(fk, oracle, pool, only=None):
         add("C3_batch50_224x224_split", lambda i: calls3[i % k3](), n * 224 * 224, alg3, "transform_kernel<ResizeJob<uchar3 -> float3 planes, N = 50>>", k3,
             verify_c3, "crops of 16..512 pixels a side at uniform positions inside 50 different 1920x1080 images")
 
-    # ---- C4: resize 4K -> 1280x720, 32 tiles of 128x128 (BASELINE configuration 4) -----------------------------------
+    # ---- C4: resize 4K -> 1280x720, 32 tiles of 128x128 (benchmark configuration 4) -----------------------------------
     if want("C4_resize_crop_32x128x128"):
         rects4 = [(160 * i, 180 * j, 128, 128) for j in range(4) for i in range(8)]
         alg4 = 32 * 383 * 383 * 3 + 32 * 128 * 128 * 12
@@ -372,7 +372,7 @@ def build_workloads(fk, oracle, pool, only=None):
             "transform_kernel<ResizeJob<uchar3 -> float3, CONDITIONAL_WITH_DEFAULT, N = 8>>", kk, verify_k1,
             "five planes are resized, three receive the default value")
 
-    # ---- C5: four chains over one 8192x8192 uchar4 image in one launch (BASELINE configuration 5) --------------------
+    # ---- C5: four chains over one 8192x8192 uchar4 image in one launch (benchmark configuration 5) --------------------
     if want("C5_divergent4_8192x8192"):
         big = pool.device_copies(5, (8192, 8192, 4), 1)[0]
         gray = torch.empty((8192, 8192), dtype=torch.uint8, device="cuda")
@@ -416,7 +416,7 @@ def cpu_baseline(binding, budget_s=10.0):
 
 
 def depth_sweep(fk, oracle, timer, steps):
-    """BASELINE configuration 2: the fused chain at each depth against the same operations as separate launches.
+    """benchmark configuration 2: the fused chain at each depth against the same operations as separate launches.
     From 32 operations on, the vector units (no FMA contraction, by design) are busy for more than half of the launch and
     lengthen it: the entry then says that they bound it, and every entry carries the fraction of the vector peak beside
     the HBM figure."""
