@@ -197,6 +197,15 @@ def test_staged_parameter_block_path(oracle):
         "out = torch.full((n, 24, 40, 3), float('nan'), device='cuda')\n"
         "for _ in range(3): fk.crop_resize_muls_bgr_tensor(torch.from_numpy(src).cuda(), rects, out, *args)\n"
         "torch.cuda.synchronize(); assert out.cpu().numpy().tobytes() == want.tobytes()\n"
+        # more launches in flight than the staging ring has slots, different jobs in turn, on two streams
+        "rects2 = [(r[0] // 2, r[1] // 2, r[2], r[3]) for r in rects]\n"
+        "want2 = o.crop_resize_muls_bgr_tensor(src, rects2, (40, 24), *args)\n"
+        "d_src = torch.from_numpy(src).cuda(); outs = [torch.full((n, 24, 40, 3), float('nan'), device='cuda') for _ in range(40)]\n"
+        "side = torch.cuda.Stream(); torch.cuda.synchronize()\n"
+        "for i, t in enumerate(outs):\n"
+        "    fk.crop_resize_muls_bgr_tensor(d_src, rects2 if i % 2 else rects, t, *args, stream=side.cuda_stream if i % 4 >= 2 else None)\n"
+        "torch.cuda.synchronize()\n"
+        "for i, t in enumerate(outs): assert t.cpu().numpy().tobytes() == (want2 if i % 2 else want).tobytes(), i\n"
         "f = o.unit_floats(2, (64, 1024, 3)); d = torch.empty((64, 1024, 3), device='cuda')\n"
         "fk.muladd_chain_f32c3(torch.from_numpy(f).cuda(), d, 64, 1.0001, 1e-4); torch.cuda.synchronize()\n"
         "assert d.cpu().numpy().tobytes() == o.muladd_chain_f32c3(f, 64, 1.0001, 1e-4).tobytes()\n"
