@@ -52,6 +52,7 @@ CAPI_SIGNATURES = {
     "fk_rgba2bgr_sub_u8c4_f32c3": [_vp, _i, _i, _sz, _f, _vp, _sz, _vp],
     "fk_divergent4_u8c4": [_vp, _i, _i, _sz, _vp, _i, _i, _f, _vp, Rect, _i, _vp, _f, _vp, _vp],
     "fk_batch_crop_cast_tensor": [_vp, _i, _i, _sz, _rp, _i, _i, _i, _vp, _vp],
+    "fk_batch_windows_saturate_muls_f32": [_vp, _i, _i, _sz, _rp, _i, _f, _f, _f, _vp, _vp],
     "fk_read_yuv": [_i, _vp, _sz, _i, _i, _vp, _sz, _vp],
     "fk_write_yuv": [_i, _vp, _sz, _i, _i, _vp, _sz, _vp],
     "fk_yuv_to_rgb": [_i, _i, _i, _i, _i, _vp, _sz, _i, _i, _vp, _sz, _vp],
@@ -299,6 +300,20 @@ def batch_crop_cast_tensor(src, rects, out, stream=None, defer=False):
     n, mh, mw, _ = out.shape
     assert n == len(rects) and out.is_contiguous()
     _deferred = _call(capi.fk_batch_crop_cast_tensor, (p, w, h, pitch, _rects(rects), n, mw, mh, C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def batch_windows_saturate_muls_f32(src, rects, out, mul_v, sub_v, div_v, stream=None, defer=False):
+    """The reference's horizontal-fusion benchmark chain. src: (H, W) uint8 whose row stride is the pitch; rects of one size;
+    out: (n, rect_h, rect_w) float32 contiguous."""
+    _, capi = load()
+    t = _dev(src, "uint8")
+    if t.dim() != 2:
+        raise FkError("expected a (h, w) image of bytes")
+    out = _dev(out, "float32")
+    assert out.shape == (len(rects), rects[0][3], rects[0][2]) and out.is_contiguous()
+    _deferred = _call(capi.fk_batch_windows_saturate_muls_f32, (C.c_void_p(t.data_ptr()), t.shape[1], t.shape[0], t.stride(0), _rects(rects), len(rects),
+                                                                float(mul_v), float(sub_v), float(div_v), C.c_void_p(out.data_ptr()), _stream(stream)), defer)
     return _deferred if defer else out
 
 

@@ -101,6 +101,25 @@ void crops_pipeline(Stream& stream, const void* src, int w, int h, size_t pitch,
     });
 }
 
+void windows_pipeline(Stream& stream, const void* src, int w, int h, size_t pitch, const fk_rect* rects, int n, float mul_v, float sub_v, float div_v,
+                      float* out) {
+    const auto read = PerThreadRead<ND::_2D, uchar>::build(view2d<uchar>(src, w, h, pitch));
+    const auto plane = [&](const fk_rect& r) {
+        return read.then(Crop<>::build(rect_of(r)))
+            .then(SaturateCast<uchar, float>::build())
+            .then(Mul<float>::build(mul_v))
+            .then(Sub<float>::build(sub_v))
+            .then(Div<float>::build(div_v));
+    };
+    std::vector<decltype(plane(rects[0]))> planes;
+    for (int i = 0; i < n; ++i) planes.push_back(plane(rects[i]));
+    const int rw = rects[0].width, rh = rects[0].height;
+    const size_t plane_floats = static_cast<size_t>(rw) * rh;
+    launch_planes(stream, planes, [&](size_t first, size_t count) {
+        return TensorWrite<float>::build(view3d<float>(out + first * plane_floats, rw, rh, static_cast<int>(count), 1));
+    });
+}
+
 // read -> Mul -> Add -> Mul -> ... (DEPTH operations) -> write, built one .then() at a time
 template <int DEPTH, int K = 0, typename Sender, typename Receiver>
 void muladd_chain(Stream& stream, const Sender& sender, float mul_v, float add_v, const Receiver& receiver) {
@@ -295,6 +314,20 @@ int fk_batch_crop_cast_tensor(const void* src, int src_w, int src_h, size_t src_
     return guarded([&]() -> int {
         Stream s(stream);
         crops_pipeline(s, src, src_w, src_h, src_pitch, rects, n, max_w, max_h, out);
+        return FK_OK;
+    });
+}
+
+int fk_batch_windows_saturate_muls_f32(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n, float mul_v,
+                                       float sub_v, float div_v, float* out, void* stream) {
+    if (src == nullptr || out == nullptr || rects == nullptr || n <= 0) return bad_argument("null pointer or no planes");
+    if (!rects_inside(rects, n, src_w, src_h)) return bad_argument("window outside the source image");
+    for (int i = 0; i < n; ++i) {
+        if (rects[i].width != rects[0].width || rects[i].height != rects[0].height) return bad_argument("every window must have the size of the first");
+    }
+    return guarded([&]() -> int {
+        Stream s(stream);
+        windows_pipeline(s, src, src_w, src_h, src_pitch, rects, n, mul_v, sub_v, div_v, out);
         return FK_OK;
     });
 }

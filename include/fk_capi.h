@@ -106,6 +106,13 @@ int fk_divergent4_u8c4(const void* src, int w, int h, size_t src_pitch, void* gr
 int fk_batch_crop_cast_tensor(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n,
                               int max_w, int max_h, float* out, void* stream);
 
+/* The reference's horizontal-fusion benchmark chain (benchmarks/fusion/benchmark_horizontal_fusion.h:55-72): a batch of
+ * n windows of one uchar image, all of the size of the first (there Ptr2D::crop at (i, i), 60 x 120, batch 1 ... 46,
+ * "120 in the paper") -> SaturateCast<uchar,float> -> Mul<float> -> Sub<float> -> Div<float> -> TensorWrite<float>, one
+ * launch per 64 planes.  out: n x rects[0].height x rects[0].width floats.  Any n >= 1. */
+int fk_batch_windows_saturate_muls_f32(const void* src, int src_w, int src_h, size_t src_pitch, const fk_rect* rects, int n,
+                                       float mul_v, float sub_v, float div_v, float* out, void* stream);
+
 /* ---- less common chain shapes ---------------------------------------------------------------------------------- */
 
 /* executeOperations(std::array<Ptr2D<uchar3>, BATCH> input, activeBatch, defaultValue, Tensor<uchar3> output, stream)

@@ -440,6 +440,14 @@ class _Lib:
                                                               self._pointers(outs), _sz(outs[0].strides[0])))
         return outs
 
+    def batch_windows_saturate_muls_f32(self, src, rects, mul_v, sub_v, div_v):
+        """src: (h, w) uint8, rects of one size -> (n, rh, rw) float32."""
+        h, w = src.shape
+        out = np.empty((len(rects), rects[0][3], rects[0][2]), np.float32)
+        self._check(self._paths_fn("batch_windows_saturate_muls_f32")(_p(src), _i(w), _i(h), _sz(src.strides[0]), rect_array(rects), _i(len(rects)),
+                                                                       _f(mul_v), _f(sub_v), _f(div_v), _p(out)))
+        return out
+
     def tensor_mul_f32c3(self, src, mul):
         """src: (planes, h, w, 3) float32 -> same shape."""
         planes, h, w, _ = src.shape

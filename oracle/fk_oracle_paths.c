@@ -90,3 +90,29 @@ int fko_tensor_mul_f32c3(const float* src, int w, int h, int planes, const float
     }
     return 0;
 }
+
+/* benchmark_horizontal_fusion.h:66-72: per element ((float)v * mul - sub) / div, each operation rounded to float
+ * (SaturateCast<uchar,float> is the plain conversion: saturate.h:35-53 clamps nothing for a wider output type). */
+int fko_batch_windows_saturate_muls_f32(const uint8_t* src, int w, int h, size_t pitch, const fko_rect* rects, int n, float mul_v, float sub_v,
+                                        float div_v, float* out) {
+    if (n <= 0) return 1;
+    for (int i = 0; i < n; ++i) {
+        const fko_rect r = rects[i];
+        if (r.x < 0 || r.y < 0 || r.width <= 0 || r.height <= 0 || r.x + r.width > w || r.y + r.height > h) return 1;
+        if (r.width != rects[0].width || r.height != rects[0].height) return 1;
+    }
+    const int rw = rects[0].width, rh = rects[0].height;
+    for (int z = 0; z < n; ++z) {
+        for (int y = 0; y < rh; ++y) {
+            const uint8_t* row = src + (size_t)(rects[z].y + y) * pitch + rects[z].x;
+            float* o = out + ((size_t)z * rh + y) * rw;
+            for (int x = 0; x < rw; ++x) {
+                const float v = (float)row[x];
+                const float m = v * mul_v;
+                const float d = m - sub_v;
+                o[x] = d / div_v;
+            }
+        }
+    }
+    return 0;
+}

@@ -37,6 +37,11 @@ int fko_batch_crop_cast_images(const uint8_t* src, int w, int h, size_t pitch, c
                                size_t out_pitch);
 /* TensorRead<float3> -> Mul<float3> -> TensorWrite<float3> (memory_operations.h:139-171). */
 int fko_tensor_mul_f32c3(const float* src, int w, int h, int planes, const float mul[3], float* out);
+/* The reference's horizontal-fusion benchmark chain (benchmarks/fusion/benchmark_horizontal_fusion.h:33-92): an array of n
+ * windows of one uchar image, all of one size (there: Ptr2D::crop at (i, i), 60 x 120) -> SaturateCast<uchar,float> ->
+ * Mul<float> -> Sub<float> -> Div<float> -> TensorWrite<float>.  out: n x rect.height x rect.width floats. */
+int fko_batch_windows_saturate_muls_f32(const uint8_t* src, int w, int h, size_t pitch, const fko_rect* rects, int n, float mul_v, float sub_v,
+                                        float div_v, float* out);
 
 #ifdef __cplusplus
 }

@@ -8,6 +8,7 @@
 #include <fused_kernel/algorithms/basic_ops/cast.h>
 #include <fused_kernel/algorithms/image_processing/crop.h>
 #include <fused_kernel/algorithms/image_processing/resize.h>
+#include <fused_kernel/algorithms/image_processing/saturate.h>
 #include <fused_kernel/fused_kernel.h>
 
 #include <array>
@@ -65,6 +66,19 @@ void crop_cast_images(const uint8_t* src, int w, int h, size_t pitch, const fko_
     const auto sender = PerThreadRead<ND::_2D, uchar3>::build(raw2d<uchar3>(src, w, h, pitch)).then(Crop<>::build(crops)).then(Cast<uchar3, float3>::build());
     executeOperations<CPU>(stream, sender, PerThreadWrite<ND::_2D, float3>::build(images));
 }
+// benchmark_horizontal_fusion.h:55-72: the batch is an array of windows of one image (Ptr2D::crop there, the same pointer
+// arithmetic here), executeOperations(array, stream, ops..., TensorWrite)
+template <size_t N>
+void windows_saturate_muls(const uint8_t* src, int w, int h, size_t pitch, const fko_rect* rects, float mul_v, float sub_v, float div_v, float* out) {
+    (void)w;
+    (void)h;
+    Stream_<ParArch::CPU> stream;
+    std::array<RawPtr<ND::_2D, uchar>, N> crops;
+    for (size_t i = 0; i < N; ++i) crops[i] = raw2d<uchar>(src + static_cast<size_t>(rects[i].y) * pitch + rects[i].x, rects[i].width, rects[i].height, pitch);
+    const auto read = PerThreadRead<ND::_2D, uchar>::build(crops);
+    executeOperations<CPU>(stream, read, SaturateCast<uchar, float>::build(), Mul<float>::build(mul_v), Sub<float>::build(sub_v), Div<float>::build(div_v),
+                           TensorWrite<float>::build(raw3d<float>(out, rects[0].width, rects[0].height, static_cast<int>(N))));
+}
 } // namespace
 
 #define FOR_BATCH(n, CALL)                                  \
@@ -99,6 +113,10 @@ int fkr_muladd_midwrite_f32c3(const float* src, int w, int h, size_t src_pitch, 
 }
 int fkr_batch_crop_cast_images(const uint8_t* src, int w, int h, size_t pitch, const fko_rect* rects, int n, float* const* outs, size_t out_pitch) {
     FOR_BATCH(n, (crop_cast_images<N>(src, w, h, pitch, rects, outs, out_pitch)))
+}
+int fkr_batch_windows_saturate_muls_f32(const uint8_t* src, int w, int h, size_t pitch, const fko_rect* rects, int n, float mul_v, float sub_v,
+                                        float div_v, float* out) {
+    FOR_BATCH(n, (windows_saturate_muls<N>(src, w, h, pitch, rects, mul_v, sub_v, div_v, out)))
 }
 int fkr_tensor_mul_f32c3(const float* src, int w, int h, int planes, const float mul[3], float* out) {
     Stream_<ParArch::CPU> stream;

@@ -1,7 +1,7 @@
 """Writes tests/golden/reference_paths_vectors.npz from the REFERENCE's own headers (oracle/_ref/libfkref_paths.so,
 built by oracle/Makefile from /root/reference as it lies there; its CPU backend): batch reads with
-CONDITIONAL_WITH_DEFAULT (copy and resize), a write in the middle of a chain, a batch of output images and a tensor as
-the source.
+CONDITIONAL_WITH_DEFAULT (copy and resize), a write in the middle of a chain, a batch of output images, a tensor as
+the source and the chain of its horizontal-fusion benchmark (a batch of windows of one uchar image).
 
 Run in the build container only: `python tests/golden/make_golden_paths.py`.  The fixture holds outputs only; the inputs
 are regenerated from the seeds in CASES.  Nothing of the reference's source is stored.
@@ -22,6 +22,8 @@ CASES = {
     "midwrite": {"seed": 51, "shape": (11, 17, 3), "mul": 1.75, "add": -0.375},
     "images": {"seed": 61, "shape": (40, 50, 3), "rects": [(0, 0, 13, 9), (37, 31, 13, 9), (5, 20, 13, 9), (20, 3, 13, 9)]},
     "tensor": {"seed": 71, "shape": (3, 6, 10, 3), "mul": (0.5, 3.0, -1.25)},
+    # benchmark_horizontal_fusion.h: windows at (i, i); its own constants (1, 1, 3.2) and a set that rounds at every step
+    "windows": {"seed": 81, "shape": (48, 70), "rects": [(i, i, 23, 17) for i in range(8)], "ops": [(1.0, 1.0, 3.2), (1.4, 0.3, 255.0)]},
 }
 
 
@@ -29,7 +31,7 @@ def inputs(o, name):
     c = CASES[name]
     if name in ("copy", "resize"):
         return [o.bytes(c["seed"] + i, c["shape"]) for i in range(c["n"])]
-    if name == "images":
+    if name in ("images", "windows"):
         return o.bytes(c["seed"], c["shape"])
     n = int(np.prod(c["shape"]))
     return o.unit_floats(c["seed"], n).reshape(c["shape"])
@@ -50,6 +52,8 @@ def run(lib, o, quirk=None):
     for i, img in enumerate(lib.batch_crop_cast_images(inputs(o, "images"), CASES["images"]["rects"])):
         out[f"images_{i}"] = img
     out["tensor"] = lib.tensor_mul_f32c3(inputs(o, "tensor"), CASES["tensor"]["mul"])
+    for k, (m, s_, d) in enumerate(CASES["windows"]["ops"]):
+        out[f"windows_{k}"] = lib.batch_windows_saturate_muls_f32(inputs(o, "windows"), CASES["windows"]["rects"], m, s_, d)
     return out
 
 

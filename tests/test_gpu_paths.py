@@ -98,3 +98,26 @@ def test_argument_errors_of_these_entry_points(fk, oracle):
     with pytest.raises(fk.FkError, match="size of the first"):
         fk.batch_crop_cast_images(src, [(0, 0, 5, 5), (1, 1, 6, 5)], [torch.zeros((5, 5, 3), device="cuda"), torch.zeros((5, 5, 3), device="cuda")])
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("n", [1, 6, 46, 64, 65, 120])
+def test_horizontal_fusion_benchmark_chain(fk, oracle, n):
+    """The reference's horizontal-fusion benchmark through the C ABI at its batch sizes (1, 6, ... 46; "120 in the paper"):
+    windows of 60 x 120 at (i, i) of one uchar image -> SaturateCast -> Mul -> Sub -> Div -> tensor; its constants and a
+    set that rounds at every step."""
+    src = oracle.bytes(1300 + n, (400, 500))
+    rects = [(i, i, 60, 120) for i in range(n)]
+    for ops in ((1.0, 1.0, 3.2), (1.4, 0.5, 255.0)):
+        out = torch.full((n, 120, 60), float("nan"), device="cuda")
+        fk.batch_windows_saturate_muls_f32(dev(src), rects, out, *ops)
+        torch.cuda.synchronize()
+        assert same_bits(out.cpu().numpy(), oracle.batch_windows_saturate_muls_f32(src, rects, *ops)), (n, ops)
+
+
+def test_horizontal_fusion_benchmark_chain_argument_errors(fk):
+    src = torch.zeros((50, 50), dtype=torch.uint8, device="cuda")
+    out = torch.empty((2, 10, 10), device="cuda")
+    with pytest.raises(fk.FkError):
+        fk.batch_windows_saturate_muls_f32(src, [(45, 0, 10, 10), (0, 0, 10, 10)], out, 1.0, 1.0, 3.2)  # outside the image
+    with pytest.raises(fk.FkError, match="size of the first"):
+        fk.batch_windows_saturate_muls_f32(src, [(0, 0, 10, 10), (0, 0, 12, 10)], out, 1.0, 1.0, 3.2)  # the tensor has one plane size

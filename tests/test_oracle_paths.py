@@ -24,7 +24,7 @@ def test_reference_vectors_bit_for_bit(oracle):
     """The reference's CPU backend interpolates with its host rule (row index from x): the oracle with that rule
     reproduces every vector."""
     got = G.run(oracle, oracle, quirk=1)
-    assert set(got) == set(GOLD.files) and len(got) == 16
+    assert set(got) == set(GOLD.files) and len(got) == 18
     for name in GOLD.files:
         assert same_bits(got[name], GOLD[name]), name
 
@@ -43,6 +43,10 @@ def test_side_by_side_with_the_reference_build(oracle, reference):
             rects = [(3 * i, 5 * i, 21, 17) for i in range(n)]
             for a, b in zip(oracle.batch_crop_cast_images(src, rects), reference.batch_crop_cast_images(src, rects)):
                 assert same_bits(a, b)
+            gray = oracle.bytes(seed + 70, (40, 90))
+            windows = [(i, i, 31, 19) for i in range(n)]
+            for ops in ((1.0, 1.0, 3.2), (0.37, -4.5, 0.003)):
+                assert same_bits(oracle.batch_windows_saturate_muls_f32(gray, windows, *ops), reference.batch_windows_saturate_muls_f32(gray, windows, *ops))
         f = oracle.unit_floats(seed, 5 * 9 * 13 * 3).reshape(5, 9, 13, 3)
         assert same_bits(oracle.tensor_mul_f32c3(f, (3.0, 0.1, -7.0)), reference.tensor_mul_f32c3(f, (3.0, 0.1, -7.0)))
         for a, b in zip(oracle.muladd_midwrite_f32c3(f[0], 1.0001, 1e-4), reference.muladd_midwrite_f32c3(f[0], 1.0001, 1e-4)):
@@ -93,3 +97,17 @@ def test_batch_images_closed_form(oracle):
         assert same_bits(img, src[y:y + h, x:x + w].astype(np.float32))
     with pytest.raises(ValueError):
         oracle.batch_crop_cast_images(src, [(0, 0, 8, 6), (0, 0, 9, 6)])
+
+
+def test_windows_chain_closed_form(oracle):
+    """((float)v * mul - sub) / div with every step rounded to float, per window; the benchmark's own check: all elements of
+    an image filled with 10 give (10 * 1 - 1) / 3.2."""
+    src = oracle.bytes(400, (50, 64))
+    rects = [(i, 2 * i, 20, 12) for i in range(9)]
+    got = oracle.batch_windows_saturate_muls_f32(src, rects, 1.4, 0.5, 255.0)
+    for z, (x, y, w, h) in enumerate(rects):
+        want = (src[y:y + h, x:x + w].astype(np.float32) * np.float32(1.4) - np.float32(0.5)) / np.float32(255.0)
+        assert same_bits(got[z], want.astype(np.float32)), z
+    flat = np.full((130, 70), 10, np.uint8)
+    got = oracle.batch_windows_saturate_muls_f32(flat, [(i, i, 60, 120) for i in range(10)], 1.0, 1.0, 3.2)
+    assert np.all(got == np.float32(9.0) / np.float32(3.2))
