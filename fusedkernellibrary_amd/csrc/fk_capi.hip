@@ -23,16 +23,25 @@ using Linear = InterpolationType;
 // batch builders of the operator API do per element of their arrays), put into batch reads of a fixed capacity with n of
 // their entries in use, and launched 64 planes at a time; `receiver_for(first, count)` builds the write for planes
 // first .. first + count - 1.  The plane table travels in the kernel-argument segment like that of a batch whose size is
-// a template argument.
+// a template argument.  Every launch gets the thread grid of the whole batch (the largest width and height among all n
+// planes, batch_operations.h:153-160), so that what a plane holds beside its own window does not depend on which launch
+// it falls in.
 constexpr size_t SMALL_BATCH = 8, LARGE_BATCH = 64;
 template <typename PlaneIOp, typename ReceiverFor>
 void launch_planes(Stream& stream, const std::vector<PlaneIOp>& planes, const ReceiverFor& receiver_for) {
+    using Op = typename PlaneIOp::Operation;
+    uint box_w = 0, box_h = 0;
+    for (const PlaneIOp& plane : planes) {
+        const uint w = Op::num_elems_x(Point(0, 0, 0), plane), h = Op::num_elems_y(Point(0, 0, 0), plane);
+        box_w = w > box_w ? w : box_w;
+        box_h = h > box_h ? h : box_h;
+    }
     for (size_t first = 0; first < planes.size(); first += LARGE_BATCH) {
         const size_t count = planes.size() - first < LARGE_BATCH ? planes.size() - first : LARGE_BATCH;
         if (count <= SMALL_BATCH) {
-            executeOperations<TransformDPP<>>(stream, BatchRead<SMALL_BATCH>::build_first(&planes[first], count), receiver_for(first, count));
+            executeOperations<TransformDPP<>>(stream, BatchRead<SMALL_BATCH>::build_first(&planes[first], count, box_w, box_h), receiver_for(first, count));
         } else {
-            executeOperations<TransformDPP<>>(stream, BatchRead<LARGE_BATCH>::build_first(&planes[first], count), receiver_for(first, count));
+            executeOperations<TransformDPP<>>(stream, BatchRead<LARGE_BATCH>::build_first(&planes[first], count, box_w, box_h), receiver_for(first, count));
         }
     }
 }

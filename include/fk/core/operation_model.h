@@ -690,16 +690,18 @@ struct BatchRead<BATCH_, PP_, void, NullType> {
 
     // A batch whose number of planes is known only at run time (this library's extension: the reference fixes it with
     // BATCH, batch_operations.h:153-208): the first `count` entries of a table of BATCH planes are filled in, and the
-    // batch's thread grid has `count` planes.
+    // batch's thread grid has `count` planes.  box_w x box_h, when given, is the least extent of the thread grid: a caller
+    // that launches one batch in several parts passes the largest width and height of the whole batch, so that every part
+    // covers what the one batch would.
     template <typename IOp>
-    static inline auto build_first(const IOp* iOps, size_t count) {
+    static inline auto build_first(const IOp* iOps, size_t count, uint box_w = 0, uint box_h = 0) {
         static_assert(PP_ == PlanePolicy::PROCESS_ALL, "every plane of a run-time batch is processed");
         static_assert(isAnyReadType<IOp>, "BatchRead is made of Read or ReadBack operations");
         using Op = typename IOp::Operation;
         using Batch = BatchRead<BATCH_, PlanePolicy::PROCESS_ALL, Op>;
         typename Batch::ParamsType params{};
         count = count < BATCH_ ? count : BATCH_;
-        uint max_w = 0, max_h = 0;
+        uint max_w = box_w, max_h = box_h;
         for (size_t i = 0; i < count; ++i) {
             params.opData[i] = static_cast<const OperationData<Op>&>(iOps[i]);
             const uint w = Op::num_elems_x(Point(0, 0, 0), iOps[i]);

@@ -63,6 +63,16 @@ inline unsigned resize_wave_rows_override() {
     return rows;
 }
 
+// FK_RESIZE_PACKED_DWORDS=n sets the capacity of the resize kernel's tile of packed pixels (0: no such tiles): for
+// measurements.
+inline unsigned resize_packed_capacity() {
+    static const unsigned dwords = [] {
+        const char* env = std::getenv("FK_RESIZE_PACKED_DWORDS");
+        return env != nullptr ? static_cast<unsigned>(std::strtoul(env, nullptr, 10)) : static_cast<unsigned>(RESIZE_PACKED_DWORDS);
+    }();
+    return dwords;
+}
+
 // ---- job construction ----------------------------------------------------------------------------------------
 namespace detail {
 // operations that resample through a matrix (Warping): their taps wander over the source rows
@@ -173,7 +183,7 @@ struct JobOf {
                 const bool large = static_cast<size_t>(max_w) * max_h * count * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
                 job.flags = dwords && large ? FLAG_STREAM_STORES : 0u;
                 // tile height, grid rows and LDS layout; sets FLAG_SOURCE_TILE when some plane's tiles are worth staging
-                job.grid_y = job.plan(used, max_h, resize_wave_rows_override());
+                job.grid_y = job.plan(used, max_h, resize_wave_rows_override(), resize_packed_capacity());
                 return job;
             } else {
                 using Job = PointwiseJob<Prog, N, Out, Defaults>;
@@ -184,16 +194,42 @@ struct JobOf {
                 job.out = out;
                 constexpr size_t out_elem = Out::IS_SPLIT ? sizeof(VBase<typename Out::Pixel>) : sizeof(typename Out::Pixel);
                 constexpr size_t out_chunk = dev::chunk_bytes(Job::K * static_cast<int>(out_elem));
-                bool flatten = Access::FLATTENS && used == count;
                 for (size_t i = 0; i < used; ++i) {
                     job.plane[i].prog = ProgramOf<PlaneIOp>::make(Planes::get(sender, i));
-                    if constexpr (Access::FLATTENS) {
+                    const auto& v = job.plane[i].prog.view;
+                    max_w = v.w > max_w ? v.w : max_w;
+                    max_h = v.h > max_h ? v.h : max_h;
+                }
+                // Windows of different sizes: every plane produces the extent of the batch's thread grid, as in the
+                // reference (batch_operations.h:153-160: max width x max height for every plane; a batch that is launched in
+                // parts carries the extent of the whole batch in its grid); beside its own window a plane then holds the
+                // parent image's pixels there (zero where the parent ends).  Decided before anything that depends on a
+                // plane's extent: the alignment tests below must see the rows the plane will really produce.
+                bool ragged = false;
+                if constexpr (std::is_same_v<View, PlainView<Src>>) {
+                    if constexpr (isBatchOperation<typename Sender::Operation>) {
+                        const ActiveThreads grid = sender.getActiveThreads();
+                        max_w = static_cast<int>(grid.x) > max_w ? static_cast<int>(grid.x) : max_w;
+                        max_h = static_cast<int>(grid.y) > max_h ? static_cast<int>(grid.y) : max_h;
+                    }
+                    for (size_t i = 0; i < used; ++i) ragged = ragged || job.plane[i].prog.view.w != max_w || job.plane[i].prog.view.h != max_h;
+                    if (ragged) {
+                        for (size_t i = 0; i < used; ++i) {
+                            job.plane[i].prog.view.w = max_w;
+                            job.plane[i].prog.view.h = max_h;
+                        }
+                    }
+                }
+                bool flatten = Access::FLATTENS && used == count && !ragged;
+                if constexpr (Access::FLATTENS) {
+                    for (size_t i = 0; i < used; ++i) {
                         const auto& v = job.plane[i].prog.view;
                         flatten = flatten && v.ox == 0 && v.oy == 0 && v.w == v.img_w && v.h > 1 &&
                                   v.pitch == static_cast<uint>(v.w) * sizeof(Src) && out.pitch == static_cast<uint>(v.w) * out_elem &&
                                   static_cast<size_t>(v.w) * v.h < (1u << 30);
                     }
                 }
+                if (flatten) max_w = max_h = 0; // found again below, from the flattened planes
                 for (size_t i = 0; i < used; ++i) {
                     auto& v = job.plane[i].prog.view;
                     if constexpr (Access::FLATTENS) {
@@ -210,23 +246,9 @@ struct JobOf {
                     if constexpr (Out::IS_SPLIT) vec = vec && out.chan_stride % out_chunk == 0;
                     // outputs larger than the caches are written with streaming stores
                     const bool stream = static_cast<size_t>(v.w) * v.h * count * sizeof(typename Out::Pixel) >= STREAM_STORE_MIN_BYTES;
-                    job.plane[i].flags = (vec ? FLAG_VECTOR_IO : 0u) | (vec && stream ? FLAG_STREAM_STORES : 0u);
+                    job.plane[i].flags = (vec ? FLAG_VECTOR_IO : 0u) | (vec && stream ? FLAG_STREAM_STORES : 0u) | (ragged ? FLAG_WHOLE_BOX : 0u);
                     max_w = v.w > max_w ? v.w : max_w;
                     max_h = v.h > max_h ? v.h : max_h;
-                }
-                if constexpr (std::is_same_v<View, PlainView<Src>>) {
-                    // Windows of different sizes: every plane produces the extent of the largest, as the reference's
-                    // thread grid does (batch_operations.h:153-160: max width x max height for every plane); beside its
-                    // own window a plane then holds the parent image's pixels there (zero where the parent ends).
-                    bool ragged = false;
-                    for (size_t i = 0; i < used; ++i) ragged = ragged || job.plane[i].prog.view.w != max_w || job.plane[i].prog.view.h != max_h;
-                    if (ragged) {
-                        for (size_t i = 0; i < used; ++i) {
-                            job.plane[i].prog.view.w = max_w;
-                            job.plane[i].prog.view.h = max_h;
-                            job.plane[i].flags |= FLAG_WHOLE_BOX;
-                        }
-                    }
                 }
                 // thread columns per block: enough to span the widest row, at most the whole block
                 const unsigned groups = ceil_div(static_cast<unsigned>(max_w), Job::K);

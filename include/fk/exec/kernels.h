@@ -62,6 +62,12 @@ __device__ __attribute__((always_inline)) inline void stream_store_at(const __am
     else if constexpr (ND == 3) __builtin_amdgcn_raw_buffer_store_b96(v, buffer, lane_offset, wave_offset, STREAM_POLICY);
     else __builtin_amdgcn_raw_buffer_store_b128(v, buffer, lane_offset, wave_offset, STREAM_POLICY);
 }
+// Range-checked loads through a buffer descriptor: a lane whose byte offset lies at or past `bytes` receives zero instead
+// of faulting.  For boxes of an image that are fetched in aligned pieces, some of which may reach past the image's last
+// row or lie past its last column.
+__device__ __attribute__((always_inline)) inline __amdgpu_buffer_rsrc_t image_buffer(const void* wave_uniform_base, const unsigned bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(wave_uniform_base), 0, static_cast<int>(bytes), 0x00020000);
+}
 // the same address in every lane, for the compiler to see
 __device__ __attribute__((always_inline)) inline char* wave_uniform(char* p) {
     const size_t a = reinterpret_cast<size_t>(p);
@@ -315,6 +321,19 @@ __device__ __attribute__((always_inline)) inline void store_group_either(const b
         store_group<K>(out, x0, y, z, v);
     }
 }
+// a pixel of three one-byte channels in the low three bytes of a dword, and back
+template <typename P>
+__device__ __attribute__((always_inline)) inline P unpack3(const unsigned int w) {
+    static_assert(sizeof(P) == 3 && cn<P> == 3, "three one-byte channels");
+    using B = VBase<P>;
+    return P{ static_cast<B>(static_cast<unsigned char>(w)), static_cast<B>(static_cast<unsigned char>(w >> 8)), static_cast<B>(static_cast<unsigned char>(w >> 16)) };
+}
+template <typename P>
+__device__ __attribute__((always_inline)) inline unsigned int pack3(const P& p) {
+    static_assert(sizeof(P) == 3 && cn<P> == 3, "three one-byte channels");
+    return static_cast<unsigned int>(static_cast<unsigned char>(p.x)) | static_cast<unsigned int>(static_cast<unsigned char>(p.y)) << 8 |
+           static_cast<unsigned int>(static_cast<unsigned char>(p.z)) << 16;
+}
 } // namespace dev
 
 // Pixels per thread: the smallest power of two that makes the wider side a whole number of 16-byte transactions and
@@ -363,6 +382,30 @@ struct SourceAccess<PlainView<T>> {
         constexpr size_t chunk = dev::chunk_bytes(K * static_cast<int>(sizeof(T)));
         const size_t first = reinterpret_cast<size_t>(v.data) + static_cast<size_t>(v.oy) * v.pitch + static_cast<size_t>(v.ox) * sizeof(T);
         return first % chunk == 0 && (v.h == 1 || v.pitch % chunk == 0);
+    }
+    // ---- quads: pixels 4q .. 4q + 3 of a row of the PARENT image, fetched as the whole dwords they occupy ----
+    // Three-byte pixels: a quad is twelve bytes, three dwords, when the image starts at a whole dword and its rows are a
+    // whole number of dwords apart.
+    static constexpr bool HAS_QUADS = sizeof(T) == 3 && alignof(T) == 1;
+    using Quad = dev::u32x3;
+    // bytes of the parent image from its first pixel to its last, up to the end of the last dword that holds one of them
+    static size_t quad_extent(const View& v) {
+        return ((static_cast<size_t>(v.img_h) - 1u) * v.pitch + static_cast<size_t>(v.img_w) * sizeof(T) + 3u) & ~static_cast<size_t>(3);
+    }
+    static bool quads_aligned(const View& v) { return reinterpret_cast<size_t>(v.data) % 4 == 0 && v.pitch % 4 == 0; }
+    __device__ __attribute__((always_inline)) static inline __amdgpu_buffer_rsrc_t quad_buffer(const View& v) {
+        const unsigned bytes = ((static_cast<unsigned>(v.img_h) - 1u) * v.pitch + static_cast<unsigned>(v.img_w) * static_cast<unsigned>(sizeof(T)) + 3u) & ~3u;
+        return dev::image_buffer(v.data, bytes);
+    }
+    __device__ __attribute__((always_inline)) static inline Quad load_quad(const __amdgpu_buffer_rsrc_t image, const View& v, const int q, const int py) {
+        return __builtin_amdgcn_raw_buffer_load_b96(image, static_cast<unsigned>(py) * v.pitch + static_cast<unsigned>(q) * 12u, 0, 0);
+    }
+    // the four pixels, each in the low three bytes of a dword
+    __device__ __attribute__((always_inline)) static inline void quad_pixels(const Quad& w, unsigned int* px) {
+        px[0] = w.x;
+        px[1] = __builtin_amdgcn_alignbyte(w.y, w.x, 3u);
+        px[2] = __builtin_amdgcn_alignbyte(w.z, w.y, 2u);
+        px[3] = w.z >> 8u;
     }
 };
 
@@ -428,6 +471,57 @@ struct SourceAccess<YuvView<PF>> {
         const size_t first = reinterpret_cast<size_t>(v.data) + (Layout::semi_planar ? 1 : 2) * static_cast<size_t>(v.ox) * sizeof(Base);
         return (v.ox & 1) == 0 && first % chunk == 0 && v.pitch % chunk == 0;
     }
+    // ---- quads: pixels 4q .. 4q + 3 of a row of the parent image (8-bit formats) ----
+    // 4:2:0 semi-planar: the four luma samples are one dword and the two chroma pairs that cover them another, at the same
+    // byte offset of the chroma row; packed 4:2:2: two dwords of one row.
+    static constexpr bool quads_supported() {
+        if constexpr (sizeof(Base) != 1) return false;
+        else if constexpr (Layout::semi_planar) return Layout::row_shift == 1;
+        else return true;
+    }
+    static constexpr bool HAS_QUADS = quads_supported();
+    using Quad = dev::u32x2;
+    static constexpr unsigned rows_of(const unsigned img_h) { return Layout::semi_planar ? img_h + ((img_h + 1u) >> 1) : img_h; }
+    static constexpr unsigned row_bytes_of(const unsigned img_w) { return Layout::semi_planar ? ((img_w + 1u) & ~1u) : 2u * ((img_w + 1u) & ~1u); }
+    static size_t quad_extent(const View& v) {
+        return ((static_cast<size_t>(rows_of(static_cast<unsigned>(v.img_h))) - 1u) * v.pitch + row_bytes_of(static_cast<unsigned>(v.img_w)) + 3u) & ~static_cast<size_t>(3);
+    }
+    static bool quads_aligned(const View& v) { return reinterpret_cast<size_t>(v.data) % 4 == 0 && v.pitch % 4 == 0; }
+    __device__ __attribute__((always_inline)) static inline __amdgpu_buffer_rsrc_t quad_buffer(const View& v) {
+        const unsigned bytes = ((rows_of(static_cast<unsigned>(v.img_h)) - 1u) * v.pitch + row_bytes_of(static_cast<unsigned>(v.img_w)) + 3u) & ~3u;
+        return dev::image_buffer(v.data, bytes);
+    }
+    __device__ __attribute__((always_inline)) static inline Quad load_quad(const __amdgpu_buffer_rsrc_t image, const View& v, const int q, const int py) {
+        Quad w;
+        if constexpr (Layout::semi_planar) {
+            const unsigned at = static_cast<unsigned>(q) * 4u;
+            w.x = __builtin_amdgcn_raw_buffer_load_b32(image, static_cast<unsigned>(py) * v.pitch + at, 0, 0);
+            w.y = __builtin_amdgcn_raw_buffer_load_b32(image, (static_cast<unsigned>(v.img_h) + (static_cast<unsigned>(py) >> 1)) * v.pitch + at, 0, 0);
+        } else {
+            w = __builtin_amdgcn_raw_buffer_load_b64(image, static_cast<unsigned>(py) * v.pitch + static_cast<unsigned>(q) * 8u, 0, 0);
+        }
+        return w;
+    }
+    // the four {Y, U, V} pixels, each in the low three bytes of a dword
+    __device__ __attribute__((always_inline)) static inline void quad_pixels(const Quad& w, unsigned int* px) {
+        if constexpr (Layout::semi_planar) {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const unsigned luma = (w.x >> (8 * k)) & 0xFFu;
+                const unsigned pair = (w.y >> (16 * (k >> 1))) & 0xFFFFu; // bytes 2 * (k / 2), 2 * (k / 2) + 1 of the chroma dword
+                const unsigned cu = (pair >> (8 * Layout::u)) & 0xFFu, cv = (pair >> (8 * Layout::v)) & 0xFFu;
+                px[k] = luma | cu << 8 | cv << 16;
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const unsigned four = k < 2 ? w.x : w.y; // the samples of pixels 2 * (k / 2), 2 * (k / 2) + 1
+                const unsigned luma = (four >> (8 * ((k & 1) ? Layout::y1 : Layout::y0))) & 0xFFu;
+                const unsigned cu = (four >> (8 * Layout::u)) & 0xFFu, cv = (four >> (8 * Layout::v)) & 0xFFu;
+                px[k] = luma | cu << 8 | cv << 16;
+            }
+        }
+    }
 };
 
 // ---- planes that only receive a value ----------------------------------------------------------------------------
@@ -454,7 +548,7 @@ __device__ __attribute__((always_inline)) inline void fill_default(const Out& ou
 } // namespace dev
 
 // ---- pointwise ---------------------------------------------------------------------------------------------------
-enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_WHOLE_BOX = 8u };
+enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_WHOLE_BOX = 8u, FLAG_PACKED_TILE = 16u, FLAG_OFFSETS_32 = 32u };
 
 template <typename Prog, size_t N, typename Out, typename Defaults = NoDefaultPlanes>
 struct PointwiseJob {
@@ -640,6 +734,12 @@ constexpr int RESIZE_TILE_W = 64;
 constexpr int RESIZE_GROUP_ROWS = 4;      // rows that a wave finishes, and writes, at a time
 constexpr int RESIZE_MAX_WAVE_ROWS = 16;
 constexpr int RESIZE_LDS_DWORDS = 6144;   // source tile capacity (24 KiB)
+// Capacity of a tile of packed three-byte pixels (one dword each), for boxes that hold more source pixels than output
+// pixels (down-scaling): 40 KiB, four such blocks per CU.
+#ifndef FK_RESIZE_PACKED_DWORDS
+#define FK_RESIZE_PACKED_DWORDS 10240
+#endif
+constexpr int RESIZE_PACKED_DWORDS = FK_RESIZE_PACKED_DWORDS;
 // A taller tile is chosen only while the grid keeps this many blocks (measured: five planes of 1920 x 1080 are slower as
 // 2550 tiles of 64 x 64 than as 5100 of 64 x 32), and only when every plane's tiles are staged in LDS.
 constexpr size_t RESIZE_MIN_BLOCKS_16 = 4096, RESIZE_MIN_BLOCKS_8 = 1024;
@@ -735,12 +835,25 @@ struct ResizeJob {
     static_assert(sizeof(Tap) % 4 == 0, "a tap is whole dwords");
     static constexpr int SLOT = static_cast<int>(sizeof(Tap)) / 4; // dwords of a source pixel in the tile
     static constexpr bool READ_IN_PLACE = N > 1;
+    // Three-byte pixels (as they lie in memory, or as the operations fused before the resize leave them, e.g. YUV -> RGB)
+    // can also be kept in the tile as one dword each.  Such a tile is filled from aligned pieces of the parent image's
+    // rows, four pixels per lane and load, all of a box's loads in flight together; it serves the boxes that the tile of
+    // float taps does not (down-scaling: more source pixels than output pixels), whose taps would otherwise be gathered
+    // from memory one pixel per lane and load, and computed (YUV -> RGB) once per tap instead of once per source pixel.
+    static constexpr bool PACKABLE = sizeof(Src) == 3 && alignof(Src) == 1 && sizeof(typename SrcView::Pixel) == 3 && Access::HAS_QUADS;
+    // dwords of a pixel in such a tile: pixels as they lie in memory stay one dword (nothing is computed to fill the tile);
+    // pixels that are computed are kept as the float taps the blend wants
+    static constexpr int PSLOT = RAW_SOURCE ? 1 : SLOT;
+    // such a tile is filled only while its box holds at most this many source pixels per output pixel (with more, the taps
+    // that are used are a minority of the box: 3x down-scaling of 32 planes of 128x128 took 11.8 us with tiles, 6.2 us with
+    // the taps read straight from memory)
+    static constexpr int PACKED_MAX_RATIO = 4;
     Prog plane[N];
     Out out;
     unsigned grid_x, grid_y;
-    // FLAG_STREAM_STORES: large output whose rows start at whole dwords; FLAG_SOURCE_TILE: some plane's tiles are worth
-    // staging in LDS, which decides how much LDS the launch asks for (a divergent launch shares one LDS size between all
-    // its jobs).
+    // FLAG_STREAM_STORES: large output whose rows start at whole dwords; FLAG_SOURCE_TILE / FLAG_PACKED_TILE: some plane's
+    // tiles are staged in LDS, as float taps / as packed pixels, which decides how much LDS the launch asks for (a
+    // divergent launch shares one LDS size between all its jobs).
     unsigned flags;
     // Rows of the tile that each of the block's four waves computes (4, 8 or 16: the tile is 64 x 4 * wave_rows).
     // What a wave does once (the tile's source box, its lanes' columns) is shared by more rows in a taller tile; a
@@ -750,7 +863,7 @@ struct ResizeJob {
     // many blocks a CU holds.  tile_dwords is the room for a source tile (a tile that needs more reads its taps directly).
     unsigned tile_dwords;
     Defaults defaults;
-    size_t lds_bytes() const { return (flags & FLAG_SOURCE_TILE) != 0u ? static_cast<size_t>(tile_dwords) * 4 + 16 : 0; }
+    size_t lds_bytes() const { return (flags & (FLAG_SOURCE_TILE | FLAG_PACKED_TILE)) != 0u ? static_cast<size_t>(tile_dwords) * 4 + 16 : 0; }
     int tile_h() const { return (BLOCK_THREADS / 64) * static_cast<int>(wave_rows); }
     // dwords a tile of a plane with these factors takes when staged, 0 when it is not worth staging (same rule as the
     // kernel applies per tile)
@@ -762,9 +875,24 @@ struct ResizeJob {
         const bool worth = rows * (cols | 1) * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * RESIZE_TILE_W * tile_h + 256;
         return worth ? static_cast<unsigned>(rows * (cols | 1) * SLOT) : 0u;
     }
+    // whether the byte offset of every pixel of a window, from the window's first pixel, fits 32 bits (with room for the
+    // few bytes that an access adds)
+    static bool window_fits_32_bits(const SrcView& s) {
+        const size_t rows = s.h > 0 ? static_cast<size_t>(s.h) : 1u, cols = s.w > 0 ? static_cast<size_t>(s.w) : 0u;
+        return (rows - 1u) * s.pitch + cols * sizeof(Src) + 16u < (static_cast<size_t>(1) << 32);
+    }
+    // dwords of a tile of packed pixels for a plane with these factors (an upper bound of what any of its tiles needs), 0
+    // when such a tile is not possible: `cols` pixels of a row lie in at most (cols + 6) / 4 aligned groups of four
+    static unsigned packed_tile_dwords(float fx, float fy, int tile_h, unsigned capacity) {
+        if (!(fx >= 0.f && fx <= 16.f && fy >= 0.f && fy <= 16.f)) return 0u;
+        const int cols = static_cast<int>((RESIZE_TILE_W - 1) * fx) + 3, rows = static_cast<int>((tile_h - 1) * fy) + 3;
+        const int quads = (cols + 6) / 4;
+        const unsigned need = static_cast<unsigned>(rows * quads * 4 * PSLOT);
+        return quads <= 64 && need <= capacity && rows * cols <= PACKED_MAX_RATIO * RESIZE_TILE_W * tile_h + 256 ? need : 0u;
+    }
     // Chooses the tile height and the LDS size from the factors of the first `count` planes; grid_x has been decided,
     // max_h is the tallest plane.  Returns the number of tile rows (grid_y).
-    unsigned plan(size_t count, int max_h, unsigned forced_wave_rows) {
+    unsigned plan(size_t count, int max_h, unsigned forced_wave_rows, unsigned packed_capacity = RESIZE_PACKED_DWORDS) {
         // the tallest tile that still leaves the grid enough blocks, and whose source boxes all fit the LDS
         const auto blocks = [&](unsigned wr) { return count * grid_x * ((static_cast<unsigned>(max_h) + 4u * wr - 1u) / (4u * wr)); };
         const auto staged_planes = [&](unsigned wr) {
@@ -778,12 +906,33 @@ struct ResizeJob {
         if (blocks(16) >= RESIZE_MIN_BLOCKS_16 && staged_planes(16) == count) wave_rows = 16;
         else if (blocks(8) >= RESIZE_MIN_BLOCKS_8 && staged_planes(8) == count) wave_rows = 8;
         if (forced_wave_rows == 4u || forced_wave_rows == 8u || forced_wave_rows == 16u) wave_rows = forced_wave_rows;
+        // 32-bit byte offsets from a window's first pixel to any of its pixels (the staging loop of three-byte sources and
+        // the line touches use them): only when every plane's window spans less than 4 GiB; otherwise nothing is staged
+        // or touched, and the taps are read with 64-bit row addresses
+        bool narrow = true;
+        if constexpr (RAW_SOURCE && sizeof(Src) == 3) {
+            for (size_t i = 0; i < count; ++i) narrow = narrow && window_fits_32_bits(plane[i].view.src);
+        }
         tile_dwords = 0;
+        if (!narrow) return (static_cast<unsigned>(max_h) + static_cast<unsigned>(tile_h()) - 1u) / static_cast<unsigned>(tile_h()); // no tiles: 64-bit addressed taps only
+        flags |= FLAG_OFFSETS_32;
+        bool packable = PACKABLE && packed_capacity != 0u;
+        if constexpr (PACKABLE) {
+            // (the kernel addresses a parent image with 32-bit offsets through a descriptor)
+            for (size_t i = 0; i < count; ++i) packable = packable && Access::quad_extent(plane[i].view.src) < (static_cast<size_t>(1) << 31);
+        }
         for (size_t i = 0; i < count; ++i) {
             const unsigned need = staged_tile_dwords(plane[i].view.fx, plane[i].view.fy, tile_h());
+            if (need != 0u) flags |= FLAG_SOURCE_TILE;
             tile_dwords = need > tile_dwords ? need : tile_dwords;
+            if constexpr (PACKABLE) {
+                if (need == 0u && packable && Access::quads_aligned(plane[i].view.src)) {
+                    const unsigned packed = packed_tile_dwords(plane[i].view.fx, plane[i].view.fy, tile_h(), packed_capacity);
+                    if (packed != 0u) flags |= FLAG_PACKED_TILE;
+                    tile_dwords = packed > tile_dwords ? packed : tile_dwords;
+                }
+            }
         }
-        if (tile_dwords != 0u) flags |= FLAG_SOURCE_TILE;
         return (static_cast<unsigned>(max_h) + static_cast<unsigned>(tile_h()) - 1u) / static_cast<unsigned>(tile_h());
     }
 
@@ -817,10 +966,14 @@ struct ResizeJob {
     // time.  What depends on the column alone is computed once for all the rows.  What depends on the row alone is the
     // same for the whole wave: lane i (i < wave_rows) computes it for row i and it is read from there.
     // `put(g, k, pixel)` takes the finished pixel of row g + k (g the group's first row, k = 0..3 known at compile time).
-    template <bool STAGED, bool INTERIOR, typename Put>
+    // MODE: where the taps come from: TAPS_DIRECT from memory, TAPS_FLOAT_TILE from the tile of float taps (columns from
+    // sx_lo, rows from sy_lo, `stride` pixels per row, edge copies included), TAPS_PACKED_TILE from the tile of packed pixels
+    // (column 0 is window column tile_x0, rows from sy_lo, `stride` dwords per row, only pixels that exist).
+    enum : int { TAPS_DIRECT = 0, TAPS_FLOAT_TILE = 1, TAPS_PACKED_TILE = 2 };
+    template <int MODE, bool INTERIOR, typename Put>
     __device__ __attribute__((always_inline)) static inline void sweep(const Prog& prog, const unsigned int* tile, const char* window, const int sx_lo,
-                                                                      const int sy_lo, const int stride, const int x, const int wy0, const int lane,
-                                                                      const int wave_rows, const Put& put) {
+                                                                      const int sy_lo, const int stride, const int tile_x0, const int x, const int wy0,
+                                                                      const int lane, const int wave_rows, const Put& put) {
         const View& v = prog.view;
         const SrcView& s = v.src;
         // a short tail is taken into registers once, ahead of the pixels (read in place it is fetched where it is used,
@@ -873,7 +1026,24 @@ struct ResizeJob {
         };
         static_assert(RESIZE_GROUP_ROWS == 4, "the group is written out above");
 
-        if constexpr (STAGED) {
+        if constexpr (MODE == TAPS_PACKED_TILE) {
+            // the tile holds the pixels of the window as they are: the second taps are clamped to its last column and row
+            const int x2 = x1 + 1 < s.w - 1 ? x1 + 1 : s.w - 1;
+            const int y2 = y1 + 1 < s.h - 1 ? y1 + 1 : s.h - 1;
+            const unsigned int* const column_a = tile + (x1 - tile_x0) * PSLOT;
+            const unsigned int* const column_b = tile + (x2 - tile_x0) * PSLOT;
+            const int row_a = (y1 - sy_lo) * stride * PSLOT, row_b = (y2 - sy_lo) * stride * PSLOT;
+            const auto pixel = [](const unsigned int* p) {
+                if constexpr (RAW_SOURCE) return to_tap(dev::unpack3<Src>(*p));
+                else return load_tap(p);
+            };
+            for (int g = 0; g < wave_rows; g += RESIZE_GROUP_ROWS) {
+                each_of_group([&](const auto k) {
+                    const int ra = __builtin_amdgcn_readlane(row_a, g + decltype(k)::value), rb = __builtin_amdgcn_readlane(row_b, g + decltype(k)::value);
+                    emit(g, k, pixel(column_a + ra), pixel(column_b + ra), pixel(column_a + rb), pixel(column_b + rb));
+                });
+            }
+        } else if constexpr (MODE == TAPS_FLOAT_TILE) {
             // the tile holds columns sx_lo.. and rows sy_lo.., edge copies included: no clamping here
             const unsigned int* const column = tile + (x1 - sx_lo) * SLOT;
             const int row_dwords = stride * SLOT;
@@ -984,9 +1154,11 @@ struct ResizeJob {
         const bool resamples = rx_lo <= rx_hi && ry_lo <= ry_hi;
 
         unsigned int* const tile = reinterpret_cast<unsigned int*>(lds_raw);
-        bool staged = false;
+        bool staged = false; // the tile holds float taps
+        bool packed = false; // the tile holds packed pixels
         int sx_lo = 0, sy_lo = 0;
-        int stride = 0; // source pixels per tile row
+        int stride = 0;  // source pixels per tile row
+        int tile_x0 = 0; // window column of the tile's column 0
         // window pixel (0, 0) and the byte range of a window row that belongs to the parent image (raw sources only)
         const char* const window = reinterpret_cast<const char*>(s.data) + static_cast<size_t>(s.oy) * s.pitch +
                                    static_cast<size_t>(s.ox) * sizeof(Src);
@@ -1002,8 +1174,79 @@ struct ResizeJob {
             stride = cols | 1;
             const int tile_px = (rx_hi - rx_lo + 1) * (ry_hi - ry_lo + 1);
             // staging pays off while a source pixel is used about once or more; strong down-scaling reads taps directly
-            staged = (job.flags & FLAG_SOURCE_TILE) != 0u && rows * stride * SLOT <= static_cast<int>(job.tile_dwords) && rows * cols <= 3 * tile_px + 256;
-            if (staged) {
+            staged = (job.flags & FLAG_SOURCE_TILE) != 0u && rows * stride * SLOT <= static_cast<int>(job.tile_dwords) && rows * stride * SLOT <= RESIZE_LDS_DWORDS &&
+                     rows * cols <= 3 * tile_px + 256;
+            tile_x0 = sx_lo;
+            if constexpr (PACKABLE) {
+                // A box that is not worth a tile of float taps as above (down-scaling: few taps per source pixel), of an image
+                // that starts at a whole dword with rows a whole number of dwords apart: the aligned groups of four pixels
+                // that cover the box's columns, in the rows of it that exist, each fetched by one thread with one load (two
+                // for 4:2:0 sources) through a descriptor of the whole parent image (a group that reaches past the image's
+                // last row end reads zeros there and cannot fault).  Pixels as they lie in memory are kept as one dword
+                // each; pixels that are computed (operations fused before the resize) are kept as float taps, computed once
+                // per source pixel.  Thread t takes groups t, t + 256, ... of the box (rows of `quads` groups); the loads of up
+                // to four of them are issued before the first is used, so a box costs one memory round trip.
+                const int box_px = rows * cols;
+                if (!staged && (job.flags & FLAG_PACKED_TILE) != 0u && box_px <= PACKED_MAX_RATIO * tile_px + 256 &&
+                    ((static_cast<unsigned>(reinterpret_cast<size_t>(s.data)) | s.pitch) & 3u) == 0u) {
+                    const int last_c = sx_lo + cols - 1 < s.w - 1 ? sx_lo + cols - 1 : s.w - 1; // window columns sx_lo .. last_c
+                    const int last_r = sy_lo + rows - 1 < s.h - 1 ? sy_lo + rows - 1 : s.h - 1;
+                    const int q_lo = (s.ox + sx_lo) >> 2;
+                    const int quads = ((s.ox + last_c) >> 2) - q_lo + 1, box_rows = last_r - sy_lo + 1;
+                    const int items = box_rows * quads;
+                    if (quads >= 1 && quads <= 64 && box_rows >= 1 && items * 4 * PSLOT <= static_cast<int>(job.tile_dwords)) {
+                        packed = true;
+                        stride = quads * 4;
+                        tile_x0 = 4 * q_lo - s.ox;
+                        constexpr int PASSES = 4;
+                        // item / quads as (item * m) >> 20 with m = ceil(2^20 / quads): exact for item < 2^20 / quads (16384 or more)
+                        const unsigned m = (0xFFFFFu + static_cast<unsigned>(quads)) / static_cast<unsigned>(quads);
+                        const __amdgpu_buffer_rsrc_t image = Access::quad_buffer(s);
+                        const int py0 = s.oy + sy_lo;
+                        for (int first = 0; first < items; first += BLOCK_THREADS * PASSES) { // (uniform)
+                            typename Access::Quad raw[PASSES];
+                            // (no branch between the loads: groups past the box's last repeat it, from the cache)
+#pragma unroll
+                            for (int u = 0; u < PASSES; ++u) {
+                                const int wanted = first + BLOCK_THREADS * u + tid;
+                                const int item = wanted < items ? wanted : items - 1;
+                                const int r = static_cast<int>((static_cast<unsigned>(item) * m) >> 20);
+                                raw[u] = Access::load_quad(image, s, q_lo + (item - r * quads), py0 + r);
+                            }
+#pragma unroll
+                            for (int u = 0; u < PASSES; ++u) {
+                                if (first + BLOCK_THREADS * u < items) { // (uniform: some group of this pass exists)
+                                    const int wanted = first + BLOCK_THREADS * u + tid;
+                                    const int item = wanted < items ? wanted : items - 1;
+                                    unsigned int px[4];
+                                    Access::quad_pixels(raw[u], px);
+                                    if constexpr (RAW_SOURCE) {
+                                        dev::u32x4 piece;
+                                        piece.x = px[0]; piece.y = px[1]; piece.z = px[2]; piece.w = px[3];
+                                        *reinterpret_cast<dev::u32x4*>(tile + item * 4) = piece;
+                                    } else {
+                                        unsigned int taps[4 * SLOT];
+#pragma unroll
+                                        for (int k = 0; k < 4; ++k) {
+                                            const Tap t = to_tap(dev::apply_tail(v.pre, dev::unpack3<typename SrcView::Pixel>(px[k])));
+                                            __builtin_memcpy(taps + k * SLOT, &t, sizeof(Tap));
+                                        }
+#pragma unroll
+                                        for (int k = 0; k < SLOT; ++k) {
+                                            dev::u32x4 piece;
+                                            piece.x = taps[4 * k]; piece.y = taps[4 * k + 1]; piece.z = taps[4 * k + 2]; piece.w = taps[4 * k + 3];
+                                            reinterpret_cast<dev::u32x4*>(tile + item * 4 * SLOT)[k] = piece;
+                                        }
+                                    }
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+            if (packed) {
+                // (staged above)
+            } else if (staged) {
                 // The lanes of a wave cover the box's columns, and where the box is narrow (32 columns or fewer) several
                 // of its rows side by side: lane = (row within the wave's pass, column).  The block's waves take the rows
                 // of a pass in turn.  Pixels read as they lie in memory (RAW_SOURCE): the loads of STAGE_ROWS passes are
@@ -1038,7 +1281,8 @@ struct ResizeJob {
                                 const int r = wanted < rows ? wanted : rows - 1;
                                 const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
                                 if constexpr (sizeof(Src) == 3) {
-                                    // (a window of less than 2 GiB: the row's offset fits the lane's 32 bits)
+                                    // (the row's offset from the window's first pixel fits the lane's 32 bits: the host stages
+                                    // tiles of three-byte pixels only for windows that span less than 4 GiB, FLAG_OFFSETS_32)
                                     if (rows_alike) {
                                         const unsigned int w = dev::load_dword_from_row(window, static_cast<unsigned>(sy) * s.pitch + voff);
                                         px[u].w[0] = aligned ? w : w >> 8u;
@@ -1077,7 +1321,7 @@ struct ResizeJob {
                 // (measured: eight 1920x1080 planes to 1280x720 31.3 -> 28.6 us; for larger boxes the touches cost more than
                 // they bring, 3x down-scaling 6.3 -> 7.6 us).
                 const int last_byte = s.w * static_cast<int>(sizeof(Src)) - 4; // last dword that lies wholly inside a window row
-                if (rows * cols <= 3 * tile_px + 256 && last_byte >= 0) {
+                if (rows * cols <= 3 * tile_px + 256 && last_byte >= 0 && (job.flags & FLAG_OFFSETS_32) != 0u) {
                     const int row_bytes = cols * static_cast<int>(sizeof(Src));
                     const int first_byte = sx_lo * static_cast<int>(sizeof(Src));
                     const int lines = (row_bytes + 127) / 128 + 1;
@@ -1120,11 +1364,16 @@ struct ResizeJob {
                     put(g, std::integral_constant<int, 3>{}, bar);
                 }
             } else if (staged) {
-                if (interior) sweep<true, true>(prog, tile, window, sx_lo, sy_lo, stride, x, wy0, lane, wave_rows, put);
-                else sweep<true, false>(prog, tile, window, sx_lo, sy_lo, stride, x, wy0, lane, wave_rows, put);
+                if (interior) sweep<TAPS_FLOAT_TILE, true>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                else sweep<TAPS_FLOAT_TILE, false>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+            } else if (PACKABLE && packed) {
+                if constexpr (PACKABLE) {
+                    if (interior) sweep<TAPS_PACKED_TILE, true>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                    else sweep<TAPS_PACKED_TILE, false>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                }
             } else {
-                if (interior) sweep<false, true>(prog, tile, window, sx_lo, sy_lo, stride, x, wy0, lane, wave_rows, put);
-                else sweep<false, false>(prog, tile, window, sx_lo, sy_lo, stride, x, wy0, lane, wave_rows, put);
+                if (interior) sweep<TAPS_DIRECT, true>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                else sweep<TAPS_DIRECT, false>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
             }
         };
         // One pixel per lane straight from registers: a wave's store covers 64 neighbouring pixels of a row (768

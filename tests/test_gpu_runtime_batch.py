@@ -64,11 +64,48 @@ def test_tiles_and_ragged_crops_any_batch(fk, oracle, n):
     fk.resize_crop_tiles(dev(src), (160, 120), tiles, out, (1 / 255.,) * 3)
     torch.cuda.synchronize()
     assert same_bits(out.cpu().numpy(), want), n
-    # crops of different sizes without a resize: every plane's own rectangle is written
-    rects = crops(oracle, 1000 + n, n, 400, 260, 1, 40)
+    # crops of different sizes without a resize: every plane receives the box of the largest width and height among ALL n
+    # crops (the thread grid of the one batch, also where the entry point launches it in parts of 64 planes); origins are
+    # drawn so that the box stays inside the image, where the oracle (exec_all=1) defines every element of it
+    rects = crops(oracle, 1000 + n, n, 360, 220, 1, 40)
+    box_w, box_h = max(r[2] for r in rects), max(r[3] for r in rects)
     got = torch.full((n, 40, 40, 3), -1.0, device="cuda")
     fk.batch_crop_cast_tensor(dev(src), rects, got)
     torch.cuda.synchronize()
     got = got.cpu().numpy()
-    for z, (x, y, w, h) in enumerate(rects):
-        assert same_bits(got[z, :h, :w], src[y:y + h, x:x + w].astype(np.float32)), (n, z)
+    want = np.full((n, 40, 40, 3), -1.0, np.float32)
+    want[:, :box_h, :box_w] = oracle.batch_crop_cast_tensor(src, rects, (box_w, box_h), exec_all=1)
+    assert same_bits(got, want), n
+
+
+def test_box_of_a_batch_launched_in_parts_is_the_whole_batch_s(fk, oracle):
+    """70 crops whose tallest lies in the first 64 and whose widest lies in the last 6: both launches must cover the box of
+    the largest width and the largest height of all 70."""
+    src = oracle.bytes(77, (120, 160, 3))
+    rects = [(i % 50, i % 30, 8, 6) for i in range(70)]
+    rects[3] = (10, 10, 9, 37)
+    rects[68] = (20, 5, 33, 4)
+    got = torch.full((70, 40, 40, 3), -1.0, device="cuda")
+    fk.batch_crop_cast_tensor(dev(src), rects, got)
+    torch.cuda.synchronize()
+    want = np.full((70, 40, 40, 3), -1.0, np.float32)
+    want[:, :37, :33] = oracle.batch_crop_cast_tensor(src, rects, (33, 37), exec_all=1)
+    assert same_bits(got.cpu().numpy(), want)
+
+
+def test_one_row_window_in_a_ragged_batch_with_an_odd_padded_pitch(fk, oracle):
+    """A window of one row batched with taller ones produces the rows of the largest: the wide (several pixels per thread)
+    path may only be taken where the rows below the first are aligned too.  Source rows 3 * 41 + 5 = 128 bytes apart and
+    131 bytes apart (odd)."""
+    src = oracle.bytes(78, (60, 41, 3))
+    rects = [(4, 7, 32, 1), (0, 0, 16, 9), (8, 20, 32, 5)]
+    want = np.full((3, 12, 36, 3), -3.0, np.float32)
+    want[:, :9, :32] = oracle.batch_crop_cast_tensor(src, rects, (32, 9), exec_all=1)
+    for extra in (5, 8):
+        padded = np.zeros((60, 41 * 3 + extra), np.uint8)
+        padded[:, :41 * 3] = src.reshape(60, -1)
+        view = torch.from_numpy(padded).cuda()[:, :41 * 3].view(60, 41, 3)
+        out = torch.full((3, 12, 36, 3), -3.0, device="cuda")
+        fk.batch_crop_cast_tensor(view, rects, out)
+        torch.cuda.synchronize()
+        assert same_bits(out.cpu().numpy(), want), extra
