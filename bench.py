@@ -34,7 +34,8 @@ DEPTH = 16
 MUL_V, ADD_V = 1.0001, 1e-4
 README_ARGS = (0, (0, 0, 0), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)  # PRESERVE_AR, background, mul, sub, div
 HEADLINE = "C1_scaled_5x1024x768_to_1920x1080"
-CONFIG_NAMES = ["C1_readme_60x60x5", HEADLINE, "C1_nobars_5x1024x576_to_1920x1080", f"C2_vertical_fusion_depth{DEPTH}", "C3_batch50_224x224_split",
+CONFIG_NAMES = ["C1_readme_60x60x5", HEADLINE, "C1_nobars_5x1024x576_to_1920x1080", "S0_setto_f32c3_60x60x5", "S1_setto_f32c3_1920x1080x5",
+                f"C2_vertical_fusion_depth{DEPTH}", "C3_batch50_224x224_split",
                 "C4_resize_crop_32x128x128", "Y1_nv12_4k_to_rgb_u8c3", "Y2_p010_4k_to_rgba_u16c4", "Y3_uyvy_4k_to_rgb_f32c3",
                 "Y4_nv12_crop1920x1080_to_1280x720_split", "Y5_nv12_crop640x360_to_1920x1080_split", "B1_reflect101_border64_4k_u8c3",
                 "W1_affine_rot5deg_4k_to_4k_f32c3", "W2_perspective_4k_to_1920x1080_f32c3", "R1_circular_tensor_update_8x1080p",
@@ -76,18 +77,38 @@ def spin_up(launch, seconds=None):
         torch.cuda.synchronize()
 
 
-def time_launches(timer, launch, steps, warmup):
+def percentile(sorted_values, q):
+    """Nearest-rank percentile of an ascending list."""
+    return sorted_values[min(len(sorted_values) - 1, max(0, int(math.ceil(q * len(sorted_values))) - 1))]
+
+
+def time_blocks(timer, launch, steps, warmup, blocks):
+    """`blocks` timed blocks of exactly `steps` launches each, every block bracketed by a device synchronisation on both
+    sides: per block the wall time per step and the time per launch by HIP events on the launch stream.  Returns the two
+    lists (milliseconds per step), in the order measured."""
     import torch
     spin_up(launch)
     for i in range(warmup):
         launch(i)
-    torch.cuda.synchronize()
-    timer.start()
-    for i in range(steps):
-        launch(i)
-    ms = timer.stop_ms()
-    torch.cuda.synchronize()
-    return ms / steps
+    wall, events, n = [], [], 0
+    for _ in range(blocks):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        timer.start()
+        for i in range(steps):
+            launch(n + i)
+        ev = timer.stop_ms()
+        torch.cuda.synchronize()
+        wall.append((time.perf_counter() - t0) * 1e3 / steps)
+        events.append(ev / steps)
+        n += steps
+    return wall, events
+
+
+def time_launches(timer, launch, steps, warmup, blocks=5):
+    """Median over `blocks` timed blocks of `steps` launches each, by HIP events (milliseconds per launch)."""
+    _, events = time_blocks(timer, launch, steps, warmup, blocks)
+    return percentile(sorted(events), 0.5)
 
 
 class HostPool:
@@ -201,6 +222,25 @@ def build_workloads(fk, oracle, pool, only=None):
            "4:3 crops into a 16:9 target under PRESERVE_AR: a quarter of the output is the bars beside the image")
     readme("C1_nobars_5x1024x576_to_1920x1080", [(64 * i, 48 * i, 1024, 576) for i in range(5)], (1920, 1080),
            "16:9 crops: every output pixel is resampled")
+
+    # ---- S0, S1: fk::setTo on the headline's output tensor and on the literal configuration's: launches that only store ----
+    def set_to(name, n, dst, note):
+        if not want(name):
+            return
+        alg = n * dst[0] * dst[1] * 12
+        k = sets_for(alg)
+        outs = [torch.empty((n, dst[1], dst[0], 3), device="cuda") for _ in range(k)]
+        value = (0.25, -1.5, 3.0)
+        calls = [fk.set_to_f32c3_tensor(value, outs[s], defer=True) for s in range(k)]
+
+        def verify(last):
+            got = outs[last % k].cpu().numpy()
+            assert same(got, np.broadcast_to(np.array(value, np.float32), got.shape).copy()), name + ": a fill that is not the value"
+        add(name, lambda i: calls[i % k](), n * dst[0] * dst[1], alg, "transform_kernel<GenericJob<ReadSet<float3> -> PerThreadWrite<_3D, float3>>>", k, verify, note)
+
+    set_to("S0_setto_f32c3_60x60x5", 5, (60, 60), "the launch floor of this runtime: 216 KB of stores, nothing read")
+    set_to("S1_setto_f32c3_1920x1080x5", 5, (1920, 1080),
+           "the store-only ceiling of the headline: the same 124.4 MB tensor written with the same streaming stores, nothing read or computed")
 
     # ---- C2: vertical fusion, depth 16 (benchmark configuration 2) ----------------------------------------------------
     name = f"C2_vertical_fusion_depth{DEPTH}"
@@ -455,6 +495,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--blocks", type=int, default=30,
+                    help="timed blocks of --steps launches each for the headline (the median block is reported); the other "
+                         "configurations take a third of them")
     ap.add_argument("--spinup-s", type=float, default=SPINUP_S,
                     help="seconds of untimed launches of each workload before its warm-up steps (shorter for traces)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -484,13 +527,19 @@ def main():
     pool = HostPool(oracle)
 
     def run(w):
+        # (blocks of at least 100 launches for these: the first launches after a synchronisation find the device idle, and
+        # over a block of 20 launches of a few microseconds each that start-up is a quarter of what is measured)
         big = w.alg_bytes > 1e9
-        steps, warmup = (max(3, args.steps // 4), max(1, args.warmup // 4)) if big else (args.steps, args.warmup)
-        ms = time_launches(timer, w.launch, steps, warmup)
+        steps, warmup = (max(3, args.steps // 4), max(1, args.warmup // 4)) if big else (max(100, args.steps), args.warmup)
+        blocks = max(1, args.blocks // 6) if big else max(1, args.blocks // 3)
+        _, events = time_blocks(timer, w.launch, steps, warmup, blocks)
+        events.sort()
+        ms = percentile(events, 0.5)
         checked = not args.no_verify
         if checked:
-            w.verify(steps - 1)
-        res = {"ms": ms, "gpixel_s": w.out_px / ms / 1e6, "buffer_sets": w.sets, "checked_against_oracle": checked, "roofline": w.roofline(ms)}
+            w.verify(blocks * steps - 1)
+        res = {"ms": ms, "ms_p10": percentile(events, 0.1), "ms_p90": percentile(events, 0.9), "timed_blocks": blocks, "steps_per_block": steps,
+               "gpixel_s": w.out_px / ms / 1e6, "buffer_sets": w.sets, "checked_against_oracle": checked, "roofline": w.roofline(ms)}
         if w.note:
             res["note"] = w.note
         return res
@@ -506,25 +555,23 @@ def main():
         return
 
     # ---- headline: the README pipeline, bandwidth-sized; exactly `steps` launches, device-synchronised on both sides ----
+    # `blocks` blocks of exactly `steps` launches, each with a device synchronisation on both sides; the figures are those of
+    # the median block (one block of 20 launches is half a millisecond: a single sample of it says little)
     head = build_workloads(fk, oracle, pool, only=HEADLINE)[0]
-    spin_up(head.launch)
-    for i in range(args.warmup):
-        head.launch(i)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    timer.start()
-    for i in range(args.steps):
-        head.launch(i)
-    kernel_ms = timer.stop_ms() / args.steps
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    blocks = max(1, args.blocks)
+    wall, events = time_blocks(timer, head.launch, args.steps, args.warmup, blocks)
+    wall.sort()
+    events.sort()
+    wall_ms, kernel_ms = percentile(wall, 0.5), percentile(events, 0.5)
     if not args.no_verify:
-        head.verify(args.steps - 1)  # the result of the last timed step is the real chain: two of its planes against the oracle
+        head.verify(blocks * args.steps - 1)  # the result of the last timed step is the real chain: two of its planes against the oracle
 
     out = {
         "metric": "fused pipeline Gpixel/s + achieved HBM GB/s (% of peak) on 1 MI355X",
         "value": head.out_px / wall_ms / 1e6, "unit": "Gpixel/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "spinup_s": SPINUP_S, "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "spinup_s": SPINUP_S, "timed_blocks": blocks, "ms_per_step": wall_ms, "ms_per_step_p10": percentile(wall, 0.1),
+        "ms_per_step_p90": percentile(wall, 0.9), "kernel_ms_p10": percentile(events, 0.1), "kernel_ms_p50": kernel_ms,
+        "kernel_ms_p90": percentile(events, 0.9), "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "README pipeline, bandwidth-sized: five 1024x768 crops of a 3840x2160 uchar3 frame -> Resize<INTER_LINEAR, PRESERVE_AR> to "
                                "1920x1080 -> x1.4 -> -0.5 -> /255 -> RGB2BGR -> float3 tensor 1920x1080x5, one fused launch per step, "

@@ -68,6 +68,7 @@ CAPI_SIGNATURES = {
     "fk_muladd_midwrite_f32c3": [_vp, _i, _i, _sz, _f, _f, _vp, _sz, _vp, _sz, _vp],
     "fk_batch_crop_cast_images": [_vp, _i, _i, _sz, _rp, _i, C.POINTER(C.c_void_p), _sz, _vp],
     "fk_tensor_mul_f32c3": [_vp, _i, _i, _i, _f3p, _vp, _vp],
+    "fk_set_to_f32c3_tensor": [_f3p, _vp, _i, _i, _i, _vp],
 }
 PACKED_TO_SPLIT, PACKED_TO_TRANSPOSED, SPLIT_TO_PACKED, TRANSPOSED_TO_PACKED = 0, 1, 2, 3
 ASCENDENT, DESCENDENT = 0, 1
@@ -82,7 +83,7 @@ RUNTIME_SYMBOLS = [
     "fkrt_device_count", "fkrt_set_device", "fkrt_get_device", "fkrt_stream_create", "fkrt_stream_destroy",
     "fkrt_stream_sync", "fkrt_malloc", "fkrt_malloc_pitch", "fkrt_free", "fkrt_malloc_host", "fkrt_free_host",
     "fkrt_memcpy_async", "fkrt_memcpy2d_async", "fkrt_memset_async", "fkrt_launch", "fkrt_params_upload",
-    "fkrt_params_release", "fkrt_max_kernarg_bytes", "fkrt_error_string", "fkrt_event_create", "fkrt_event_destroy",
+    "fkrt_params_release", "fkrt_max_kernarg_bytes", "fkrt_last_error", "fkrt_error_string", "fkrt_event_create", "fkrt_event_destroy",
     "fkrt_event_record", "fkrt_event_sync", "fkrt_event_elapsed_ms",
 ]
 
@@ -510,4 +511,14 @@ def tensor_mul_f32c3(src, mul, out, stream=None, defer=False):
     assert src.shape == out.shape and src.shape[3] == 3 and src.is_contiguous() and out.is_contiguous()
     planes, h, w, _ = src.shape
     _deferred = _call(capi.fk_tensor_mul_f32c3, (C.c_void_p(src.data_ptr()), w, h, planes, _f3(mul), C.c_void_p(out.data_ptr()), _stream(stream)), defer)
+    return _deferred if defer else out
+
+
+def set_to_f32c3_tensor(value, out, stream=None, defer=False):
+    """fk::setTo on a tensor of packed float3. out: (planes, H, W, 3) float32 contiguous."""
+    _, capi = load()
+    out = _dev(out, "float32")
+    assert out.dim() == 4 and out.shape[3] == 3 and out.is_contiguous()
+    planes, h, w, _ = out.shape
+    _deferred = _call(capi.fk_set_to_f32c3_tensor, (_f3(value), C.c_void_p(out.data_ptr()), w, h, planes, _stream(stream)), defer)
     return _deferred if defer else out

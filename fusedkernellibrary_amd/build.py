@@ -41,7 +41,9 @@ def _run(cmd):
 
 def build_runtime():
     out = os.path.join(HERE, "libfk_hip_rt.so")
-    _run([hipcc(), os.path.join(CSRC, "fk_hip_rt.cpp"), "-I" + INCLUDE, "-std=c++17", "-O2", "-fPIC", "-shared", "-o", out])
+    # compiled as HIP: it holds the kernel-argument probe kernel
+    _run([hipcc(), "-x", "hip", os.path.join(CSRC, "fk_hip_rt.cpp"), "-I" + INCLUDE, "--offload-arch=gfx950", "-std=c++17", "-O2",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-fPIC", "-shared", "-o", out])
     return out
 
 
@@ -78,6 +80,15 @@ def build_cpp_tests():
         _run([hipcc(), "-x", "hip", os.path.join(tests, name + ".cpp"), "-I" + INCLUDE, *DEVICE_FLAGS, "-L" + HERE, "-lfk_hip_rt",
               "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/../../fusedkernellibrary_amd", "-o", out])
         outs.append(out)
+    # host-only checks: the launch plans (no GPU call is made), and the staging ring's slot state machine with stand-ins
+    # for the GPU runtime (plain g++, no GPU header)
+    out = os.path.join(tests, "host_plan_check")
+    _run([hipcc(), "-x", "hip", "--cuda-host-only", os.path.join(tests, "host_plan_check.cpp"), "-I" + INCLUDE, "-std=c++17", "-O1",
+          "-L" + HERE, "-lfk_hip_rt", "-Wl,-rpath," + HERE, "-Wl,-rpath,$ORIGIN/../../fusedkernellibrary_amd", "-o", out])
+    outs.append(out)
+    out = os.path.join(tests, "staging_ring_check")
+    _run([shutil.which("g++") or "g++", "-std=c++17", "-O2", "-pthread", "-I" + CSRC, os.path.join(tests, "staging_ring_check.cpp"), "-o", out])
+    outs.append(out)
     return outs
 
 
@@ -90,12 +101,12 @@ def build_benchmarks():
 
 
 # The reference's own test headers that exercise this path's operator API (relative to the reference checkout); each
-# defines `int launch()`.  Left out: examples/readme_test_code.h (half of it runs on the reference's CPU backend) and
-# benchmarks/ (their timing harness is written against the CUDA runtime's event and
+# defines `int launch()`.  Left out: benchmarks/ (their timing harness is written against the CUDA runtime's event and
 # stream types; fusedkernellibrary_amd/benchmarks/reference_sweeps.cpp restates them).
 REFERENCE_TESTS = (
     "tests/algorithm/test_batchresize_build.h", "tests/algorithm/test_border_reader.h", "tests/algorithm/test_crop.h",
-    "tests/algorithm/test_deinterlace.h", "tests/algorithm/test_warp.h", "tests/data/test_ptr_nd.h", "tests/data/test_rect.h",
+    "tests/algorithm/test_deinterlace.h", "tests/algorithm/test_warp.h", "tests/data/basic_test.h", "tests/data/test_ptr_nd.h", "tests/data/test_rect.h",
+    "tests/examples/readme_test_code.h",
     "tests/data/test_tuple.h", "tests/data/test_typelist.h", "tests/operation/test_filtered_index_sequence.h",
     "tests/operation/test_fused_operation.h", "tests/operation/test_instantiable_operations.h",
     "tests/operation/test_operation_fuser.h", "tests/operation/test_operation_tuple.h", "tests/operation/test_operation_types.h",

@@ -57,8 +57,12 @@ int run(Stream& stream, void* block, const void* src, int w, int h, size_t pitch
     using PlaneIOp = decltype(readme_plane<AR>(src, w, h, pitch, rects[0], dw, dh, bg, mul, sub, div));
     PlaneIOp planes[PLANES];
     for (int i = 0; i < n; ++i) planes[i] = readme_plane<AR>(src, w, h, pitch, rects[i], dw, dh, bg, mul, sub, div);
-    const bool fits = Executor<TransformDPP<>>::executeOperationsFrom(block, SCRATCH_BYTES, stream, BatchRead<PLANES>::build_first(planes, static_cast<size_t>(n)),
-                                                                       TensorWrite<float3>::build(view3d<float3>(out, dw, dh, n, 1)));
+    const auto sender = BatchRead<PLANES>::build_first(planes, static_cast<size_t>(n));
+    const auto receiver = TensorWrite<float3>::build(view3d<float3>(out, dw, dh, n, 1));
+    // a job that outgrows the block must fail the build, not the call
+    using Job = decltype(exec::JobOf<std::decay_t<decltype(sender)>, std::decay_t<decltype(receiver)>>::make(sender, receiver));
+    static_assert(sizeof(Job) <= SCRATCH_BYTES, "the job of a full batch no longer fits FK_NOALLOC_MAX_JOB_BYTES");
+    const bool fits = Executor<TransformDPP<>>::executeOperationsFrom(block, SCRATCH_BYTES, stream, sender, receiver);
     return fits ? FK_OK : unsupported("the chain's parameters exceed the library's fixed device block (or the kernel-argument limit)");
 }
 } // namespace

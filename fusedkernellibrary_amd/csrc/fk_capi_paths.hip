@@ -120,4 +120,16 @@ int fk_tensor_mul_f32c3(const void* src, int w, int h, int planes, const float m
     });
 }
 
+int fk_set_to_f32c3_tensor(const float value[3], void* out, int w, int h, int planes, void* stream) {
+    if (out == nullptr || value == nullptr || w <= 0 || h <= 0 || planes <= 0) return bad_argument("null pointer or empty tensor");
+    return guarded([&]() -> int {
+        Stream s(stream);
+        // what fk::setTo launches for a Tensor<float3> in device memory
+        const ActiveThreads extent(static_cast<uint>(w), static_cast<uint>(h), static_cast<uint>(planes));
+        executeOperations<TransformDPP<>>(s, ReadSet<float3>::build(float3{ value[0], value[1], value[2] }, extent),
+                                          PerThreadWrite<ND::_3D, float3>::build(view3d<float3>(out, w, h, planes, 1)));
+        return FK_OK;
+    });
+}
+
 } // extern "C"

@@ -377,6 +377,19 @@ public:
     Ptr3D<T> crop3D(const Point& p, const PtrDims<ND::_3D>& newDims) { return Ptr<ND::_3D, T>::crop(p, newDims); }
 };
 
+// A 3D pointer whose channel planes are outermost (ptr_nd.h:661-675).
+template <typename T>
+class PtrT3D : public Ptr<ND::T3D, T> {
+public:
+    PtrT3D(const uint& width_, const uint& height_, const uint& planes_, const uint& color_planes_ = 1, const MemType& type_ = defaultMemType,
+           const int& deviceID_ = 0)
+        : Ptr<ND::T3D, T>(PtrDims<ND::T3D>(width_, height_, planes_, color_planes_), type_, deviceID_) {}
+    PtrT3D(const Ptr<ND::T3D, T>& other) : Ptr<ND::T3D, T>(other) {}
+    PtrT3D(T* data_, const PtrDims<ND::T3D>& dims_, const MemType& type_ = MemType::Device, const int& deviceID_ = 0)
+        : Ptr<ND::T3D, T>(data_, dims_, type_, deviceID_) {}
+    PtrT3D<T> crop3D(const Point& p, const PtrDims<ND::T3D>& newDims) { return Ptr<ND::T3D, T>::crop(p, newDims); }
+};
+
 // width x height x planes images of `color_planes` channel planes each, rows always tight.
 template <typename T>
 class Tensor : public Ptr<ND::_3D, T> {

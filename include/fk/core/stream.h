@@ -26,14 +26,23 @@ enum class ParArch {
 // This library executes on one backend only.
 constexpr ParArch defaultParArch = ParArch::GPU_AMD;
 
+// What every stream can do (core/execution_model/stream.h:29-47).
+class BaseStream {
+public:
+    BaseStream() = default;
+    BaseStream(const BaseStream&) = default;
+    BaseStream& operator=(const BaseStream&) = default;
+    virtual ~BaseStream() = default;
+    virtual void sync() = 0;
+};
+
 template <ParArch PA>
 class Stream_ {
-    static_assert(PA == ParArch::GPU_AMD,
-                  "Only ParArch::GPU_AMD is implemented by this library; there is no host fallback executor.");
+    static_assert(PA == ParArch::GPU_AMD || PA == ParArch::CPU, "Only ParArch::GPU_AMD and ParArch::CPU are implemented by this library.");
 };
 
 template <>
-class Stream_<ParArch::GPU_AMD> final {
+class Stream_<ParArch::GPU_AMD> final : public BaseStream {
     struct Owned {
         fkrt_stream handle{ nullptr };
         ~Owned() {
@@ -60,9 +69,19 @@ public:
     operator fkrt_stream() const { return m_stream; }
     fkrt_stream getHIPStream() const { return m_stream; }
     int getRefCount() const { return m_owned ? static_cast<int>(m_owned.use_count()) : 0; }
-    void sync() { gpuErrchk(fkrt_stream_sync(m_stream)); }
+    void sync() final { gpuErrchk(fkrt_stream_sync(m_stream)); }
     constexpr ParArch getParArch() const { return ParArch::GPU_AMD; }
     static constexpr ParArch parArch() { return ParArch::GPU_AMD; }
+};
+
+// The host executor runs a chain before it returns: its stream has nothing to wait for (stream.h:112-124).
+template <>
+class Stream_<ParArch::CPU> final : public BaseStream {
+public:
+    Stream_() = default;
+    void sync() final {}
+    constexpr ParArch getParArch() const { return ParArch::CPU; }
+    static constexpr ParArch parArch() { return ParArch::CPU; }
 };
 
 using Stream = Stream_<defaultParArch>;

@@ -20,8 +20,7 @@ namespace fk {
 template <ParArch PA = defaultParArch, TF TFEN = TF::DISABLED>
 struct TransformDPP {
     static constexpr ParArch PAR_ARCH = PA;
-    static_assert(PA == ParArch::GPU_AMD,
-                  "Only ParArch::GPU_AMD is implemented by this library; there is no host fallback executor.");
+    static_assert(PA == ParArch::GPU_AMD || PA == ParArch::CPU, "Only ParArch::GPU_AMD and ParArch::CPU are implemented by this library.");
 };
 
 // One fused chain per group of thread planes, all in one launch.
@@ -438,6 +437,48 @@ struct Executor<TransformDPP<ParArch::GPU_AMD, TFEN>> {
     static inline void executeOperations(const std::array<Ptr2D<I>, BATCH>& input, const Tensor<O>& output,
                                          Stream_<ParArch::GPU_AMD>& stream, const IOps&... iOps) {
         executeOperations(stream, PerThreadRead<ND::_2D, I>::build(input), iOps..., PerThreadWrite<ND::_3D, O>::build(output));
+    }
+};
+
+// The same chains on the host, for user code that asks for them by name (executors.h:147-173): one element after the other
+// in the reference's order, planes outermost then rows then columns (data_parallel_patterns.h:285-298), each through the
+// operations' own exec functions, which are the ones the generic kernel calls per element.  Memory must be host memory
+// (MemType::Host, HostPinned, or the pinned side of a buffer).  Nothing here is used by the GPU path, and the GPU path
+// never falls back to it: the executor is chosen by the ParArch that the caller names.
+template <TF TFEN>
+struct Executor<TransformDPP<ParArch::CPU, TFEN>> {
+    FK_STATIC_STRUCT(Executor, Executor)
+    static constexpr ParArch parArch() { return ParArch::CPU; }
+
+    template <typename... IOps>
+    static inline void executeOperations(Stream_<ParArch::CPU>&, const IOps&... iOps) {
+        const auto seq = buildOperationSequence(iOps...);
+        using Sender = std::decay_t<decltype(seq.sender)>;
+        using Receiver = std::decay_t<decltype(seq.receiver)>;
+        const ActiveThreads grid = seq.sender.getActiveThreads();
+        for (int z = 0; z < static_cast<int>(grid.z); ++z) {
+            for (int y = 0; y < static_cast<int>(grid.y); ++y) {
+                for (int x = 0; x < static_cast<int>(grid.x); ++x) {
+                    const Point thread(x, y, z);
+                    Receiver::Operation::exec(thread, Sender::Operation::exec(thread, seq.sender), seq.receiver);
+                }
+            }
+        }
+    }
+    // Convenience forms over buffers (executors.h:52-93); the buffers' host side is what is read and written.
+    template <ND D, typename I, typename... IOps>
+    static inline void executeOperations(const Ptr<D, I>& input, Stream_<ParArch::CPU>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<D, I>::build(host_side(input)), iOps...);
+    }
+    template <ND D, typename I, typename O, typename... IOps>
+    static inline void executeOperations(const Ptr<D, I>& input, const Ptr<D, O>& output, Stream_<ParArch::CPU>& stream, const IOps&... iOps) {
+        executeOperations(stream, PerThreadRead<D, I>::build(host_side(input)), iOps..., PerThreadWrite<D, O>::build(host_side(output)));
+    }
+
+private:
+    template <ND D, typename T>
+    static RawPtr<D, T> host_side(const Ptr<D, T>& p) {
+        return p.getMemType() == MemType::DeviceAndPinned ? p.ptrPinned() : p.ptr();
     }
 };
 

@@ -401,11 +401,17 @@ struct SourceAccess<PlainView<T>> {
         return __builtin_amdgcn_raw_buffer_load_b96(image, static_cast<unsigned>(py) * v.pitch + static_cast<unsigned>(q) * 12u, 0, 0);
     }
     // the four pixels, each in the low three bytes of a dword
-    __device__ __attribute__((always_inline)) static inline void quad_pixels(const Quad& w, unsigned int* px) {
+    __device__ __attribute__((always_inline)) static inline void quad_dwords(const Quad& w, unsigned int* px) {
         px[0] = w.x;
         px[1] = __builtin_amdgcn_alignbyte(w.y, w.x, 3u);
         px[2] = __builtin_amdgcn_alignbyte(w.z, w.y, 2u);
         px[3] = w.z >> 8u;
+    }
+    __device__ __attribute__((always_inline)) static inline void quad_pixels(const Quad& w, T* px) {
+        unsigned int d[4];
+        quad_dwords(w, d);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) px[k] = dev::unpack3<T>(d[k]);
     }
 };
 
@@ -502,23 +508,20 @@ struct SourceAccess<YuvView<PF>> {
         }
         return w;
     }
-    // the four {Y, U, V} pixels, each in the low three bytes of a dword
-    __device__ __attribute__((always_inline)) static inline void quad_pixels(const Quad& w, unsigned int* px) {
+    // the four {Y, U, V} pixels; the two pixels of a pair receive the very same chroma values, so that what is computed from
+    // the chroma alone (centring, products with the matrix) is computed once per pair
+    __device__ __attribute__((always_inline)) static inline void quad_pixels(const Quad& w, Pixel* px) {
         if constexpr (Layout::semi_planar) {
+            const Base cu[2] = { static_cast<Base>(w.y >> (8 * Layout::u)), static_cast<Base>(w.y >> (16 + 8 * Layout::u)) };
+            const Base cv[2] = { static_cast<Base>(w.y >> (8 * Layout::v)), static_cast<Base>(w.y >> (16 + 8 * Layout::v)) };
 #pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const unsigned luma = (w.x >> (8 * k)) & 0xFFu;
-                const unsigned pair = (w.y >> (16 * (k >> 1))) & 0xFFFFu; // bytes 2 * (k / 2), 2 * (k / 2) + 1 of the chroma dword
-                const unsigned cu = (pair >> (8 * Layout::u)) & 0xFFu, cv = (pair >> (8 * Layout::v)) & 0xFFu;
-                px[k] = luma | cu << 8 | cv << 16;
-            }
+            for (int k = 0; k < 4; ++k) px[k] = Pixel{ static_cast<Base>(w.x >> (8 * k)), cu[k >> 1], cv[k >> 1] };
         } else {
+            const unsigned four[2] = { w.x, w.y }; // the samples of pixels 0, 1 and of pixels 2, 3
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
-                const unsigned four = k < 2 ? w.x : w.y; // the samples of pixels 2 * (k / 2), 2 * (k / 2) + 1
-                const unsigned luma = (four >> (8 * ((k & 1) ? Layout::y1 : Layout::y0))) & 0xFFu;
-                const unsigned cu = (four >> (8 * Layout::u)) & 0xFFu, cv = (four >> (8 * Layout::v)) & 0xFFu;
-                px[k] = luma | cu << 8 | cv << 16;
+                const unsigned f = four[k >> 1];
+                px[k] = Pixel{ static_cast<Base>(f >> (8 * ((k & 1) ? Layout::y1 : Layout::y0))), static_cast<Base>(f >> (8 * Layout::u)), static_cast<Base>(f >> (8 * Layout::v)) };
             }
         }
     }
@@ -913,6 +916,7 @@ struct ResizeJob {
         if constexpr (RAW_SOURCE && sizeof(Src) == 3) {
             for (size_t i = 0; i < count; ++i) narrow = narrow && window_fits_32_bits(plane[i].view.src);
         }
+        packed_capacity = packed_capacity < static_cast<unsigned>(RESIZE_PACKED_DWORDS) ? packed_capacity : static_cast<unsigned>(RESIZE_PACKED_DWORDS);
         tile_dwords = 0;
         if (!narrow) return (static_cast<unsigned>(max_h) + static_cast<unsigned>(tile_h()) - 1u) / static_cast<unsigned>(tile_h()); // no tiles: 64-bit addressed taps only
         flags |= FLAG_OFFSETS_32;
@@ -1199,8 +1203,12 @@ struct ResizeJob {
                         stride = quads * 4;
                         tile_x0 = 4 * q_lo - s.ox;
                         constexpr int PASSES = 4;
-                        // item / quads as (item * m) >> 20 with m = ceil(2^20 / quads): exact for item < 2^20 / quads (16384 or more)
-                        const unsigned m = (0xFFFFFu + static_cast<unsigned>(quads)) / static_cast<unsigned>(quads);
+                        // item / quads as (item * m) >> 20: exact for every item below N when 2^20 / quads <= m < 2^20 / quads *
+                        // (1 + 1 / N).  The reciprocal instruction is within 2^-22 of 1 / quads, so its product with 2^20,
+                        // truncated, plus 2 lies between 2^20 / quads + 0.7 and 2^20 / quads + 2.3; with quads <= 64 and fewer
+                        // than 2560 items (a tile is 10240 dwords at most) the upper limit is 2^20 / quads + 6.4.
+                        static_assert(RESIZE_PACKED_DWORDS <= 10240, "the division by multiplication is exact for fewer than 2560 items");
+                        const unsigned m = static_cast<unsigned>(1048576.0f * __builtin_amdgcn_rcpf(static_cast<float>(quads))) + 2u;
                         const __amdgpu_buffer_rsrc_t image = Access::quad_buffer(s);
                         const int py0 = s.oy + sy_lo;
                         for (int first = 0; first < items; first += BLOCK_THREADS * PASSES) { // (uniform)
@@ -1218,17 +1226,19 @@ struct ResizeJob {
                                 if (first + BLOCK_THREADS * u < items) { // (uniform: some group of this pass exists)
                                     const int wanted = first + BLOCK_THREADS * u + tid;
                                     const int item = wanted < items ? wanted : items - 1;
-                                    unsigned int px[4];
-                                    Access::quad_pixels(raw[u], px);
                                     if constexpr (RAW_SOURCE) {
+                                        unsigned int px[4];
+                                        Access::quad_dwords(raw[u], px);
                                         dev::u32x4 piece;
                                         piece.x = px[0]; piece.y = px[1]; piece.z = px[2]; piece.w = px[3];
                                         *reinterpret_cast<dev::u32x4*>(tile + item * 4) = piece;
                                     } else {
+                                        typename SrcView::Pixel px[4];
+                                        Access::quad_pixels(raw[u], px);
                                         unsigned int taps[4 * SLOT];
 #pragma unroll
                                         for (int k = 0; k < 4; ++k) {
-                                            const Tap t = to_tap(dev::apply_tail(v.pre, dev::unpack3<typename SrcView::Pixel>(px[k])));
+                                            const Tap t = to_tap(dev::apply_tail(v.pre, px[k]));
                                             __builtin_memcpy(taps + k * SLOT, &t, sizeof(Tap));
                                         }
 #pragma unroll

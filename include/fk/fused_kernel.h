@@ -15,6 +15,7 @@
 #include "fk/ops/static_loop.h"
 #include "fk/ops/circular.h"
 #include "fk/ops/deinterlace.h"
+#include "fk/core/reference_surface.h"
 
 namespace fk {
 

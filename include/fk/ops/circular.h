@@ -299,12 +299,21 @@ struct SequenceSelectorType {
     }
 };
 
+// the struct forms behind CTReadDirection_v and CoreType_t (circular_tensor.h:37-66)
+template <CircularTensorOrder CT_ORDER>
+struct CTReadDirection {
+    static constexpr CircularDirection dir = CT_ORDER == CircularTensorOrder::NewestFirst ? CircularDirection::Descendent : CircularDirection::Ascendent;
+};
 template <CircularTensorOrder CT_ORDER>
 constexpr CircularDirection CTReadDirection_v = CT_ORDER == CircularTensorOrder::NewestFirst ? CircularDirection::Descendent : CircularDirection::Ascendent;
 
 enum class ColorPlanes { Standard, Transposed };
 template <typename T, ColorPlanes CP_MODE>
 using CoreType_t = std::conditional_t<CP_MODE == ColorPlanes::Standard, Tensor<T>, TensorT<T>>;
+template <typename T, ColorPlanes CP_MODE>
+struct CoreType {
+    using type = CoreType_t<T, CP_MODE>;
+};
 
 template <typename T, int COLOR_PLANES, typename Enabler = void>
 struct CircularTensorStoreType {};

@@ -142,6 +142,9 @@ int fk_batch_crop_cast_images(const void* src, int w, int h, size_t pitch, const
 /* TensorRead<float3> -> Mul<float3> -> TensorWrite<float3> (memory_operations.h:139-171, 173-193): planes x h x w packed
  * float3 on both sides. */
 int fk_tensor_mul_f32c3(const void* src, int w, int h, int planes, const float mul[3], void* out, void* stream);
+/* fk::setTo(value, Tensor<float3>, stream) for a tensor in device memory (core/data/ptr_utils.h:23-45): ReadSet<float3> ->
+ * PerThreadWrite<_3D,float3>, a launch that only stores.  out: planes x h x w packed float3. */
+int fk_set_to_f32c3_tensor(const float value[3], void* out, int w, int h, int planes, void* stream);
 
 /* ---- YUV front-end ------------------------------------------------------------------------------------------
  * A raw YUV image is ONE 2D allocation of base elements (uint8 for the 8-bit formats, uint16 with the sample in the

@@ -56,14 +56,23 @@ int fkrt_launch(const void* kernel, unsigned grid_x, unsigned grid_y, unsigned g
  * from host memory into a device buffer that stays valid until the work enqueued on `s` up to the matching
  * fkrt_params_release has run; call that after enqueueing the kernel that reads the block.  `host_src` is copied before
  * the call returns and may be released at once.  The buffers come from a ring of eight slots that this layer owns (a
- * pinned host buffer and a device buffer each): nothing is allocated per call, and a ninth upload waits on the host
- * until the first slot's kernel has finished.  At most eight blocks may be between their upload and their release at
- * any time (host threads that stage blocks concurrently: at most eight of them). */
+ * pinned host buffer and a device buffer each): nothing is allocated per call.  A slot is leased to its caller from the
+ * upload to the release and is handed out again only when the kernel behind the release has finished: an upload that
+ * finds no slot free waits for that kernel on the host (without blocking other callers of this layer), and an upload
+ * that finds all eight slots leased waits up to two seconds for a release and then fails with the runtime's "not ready"
+ * status rather than overwrite a block whose kernel has not run.  A block that is never released keeps its slot. */
 int fkrt_params_upload(void** device_out, const void* host_src, size_t bytes, fkrt_stream s);
 int fkrt_params_release(void* device_params, fkrt_stream s);
 
-/* Largest by-value kernel-argument block, in bytes, that launches are allowed to use. */
+/* Largest by-value kernel-argument block, in bytes, that launches are allowed to use: 32768 where the device is seen to
+ * receive such a block intact (the first call launches a one-block probe kernel whose 32 KiB argument it sums up; it
+ * allocates nothing but synchronises, so it must not be made during stream capture), else the 4096 that HIP documents.
+ * The environment variable FK_MAX_KERNARG_BYTES (>= 256) overrides both. */
 size_t fkrt_max_kernarg_bytes(void);
+
+/* Status of the last runtime call of this thread, cleared by the call (hipGetLastError; CUDA: cudaGetLastError, used by the
+ * reference's gpuErrchk after every launch, core/utils/utils.h:95-147). */
+int fkrt_last_error(void);
 
 const char* fkrt_error_string(int status);
 

@@ -18,7 +18,7 @@ def native_build():
     """The native libraries and C++ test programs: used as built; compiled here only when nothing has been built yet."""
     import fusedkernellibrary_amd as lib
     from fusedkernellibrary_amd import build
-    wanted = list(lib.library_paths()) + [os.path.join(ROOT, "tests", "cpp", n) for n in ("conformance", "readme_dropin", "api_gpu")]
+    wanted = list(lib.library_paths()) + [os.path.join(ROOT, "tests", "cpp", n) for n in ("conformance", "readme_dropin", "api_gpu", "host_plan_check", "staging_ring_check")]
     wanted.append(os.path.join(ROOT, "fusedkernellibrary_amd", "benchmarks", "reference_sweeps"))
     if not all(os.path.exists(p) for p in wanted):
         build.build_all()

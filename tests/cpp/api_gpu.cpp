@@ -463,6 +463,38 @@ int main() {
         for (uint x = 1; x < 32; ++x) varied = varied || together.at(x, 3, 150).x != together.at(0, 3, 150).x;
         EXPECT(varied);
     }
+    // 15. the README chain through the host executor (TransformDPP<ParArch::CPU>, host memory) and through the GPU executor:
+    // the same bits, on the README's own crops (up- and down-scaling, bars on either side) and on a small frame
+    {
+        constexpr size_t BATCH = 5;
+        Ptr2D<uchar3> frame(320, 200);
+        fill_ramp(frame, stream, 7);
+        Ptr2D<uchar3> host_frame(320, 200, 0, MemType::Host);
+        for (uint y = 0; y < 200; ++y)
+            for (uint x = 0; x < 320; ++x) host_frame.at(x, y) = frame.at(x, y);
+        const std::array<Rect, BATCH> crops{ Rect(0, 0, 34, 25), Rect(10, 10, 70, 15), Rect(20, 20, 60, 59), Rect(30, 30, 20, 23), Rect(40, 40, 12, 11) };
+        const auto chain = [&](const auto& image) {
+            return PerThreadRead<ND::_2D, uchar3>::build(image)
+                .then(Crop<>::build(crops))
+                .then(Resize<InterpolationType::INTER_LINEAR, AspectRatio::PRESERVE_AR>::build(Size(60, 60), float3{ 0.f, 0.f, 0.f }))
+                .then(Mul<float3>::build(make_set<float3>(1.4f)))
+                .then(Sub<float3>::build(make_set<float3>(0.5f)))
+                .then(Div<float3>::build(make_set<float3>(255.f)))
+                .then(ColorConversion<ColorConversionCodes::COLOR_RGB2BGR, float3, float3>::build());
+        };
+        Tensor<float3> on_gpu(60, 60, BATCH);
+        Tensor<float3> on_host(60, 60, BATCH, 1, MemType::Host);
+        executeOperations<TransformDPP<>>(stream, chain(frame), TensorWrite<float3>::build(on_gpu));
+        on_gpu.download(stream);
+        stream.sync();
+        Stream_<ParArch::CPU> host_stream;
+        executeOperations<TransformDPP<ParArch::CPU>>(host_stream, chain(host_frame), TensorWrite<float3>::build(on_host));
+        host_stream.sync();
+        EXPECT(std::memcmp(on_gpu.ptrPinned().data, on_host.ptr().data, on_host.sizeInBytes()) == 0);
+        bool varied = false;
+        for (uint x = 1; x < 60; ++x) varied = varied || on_host.at(x, 30, 2).x != on_host.at(0, 30, 2).x;
+        EXPECT(varied);
+    }
     // 8. a launch the runtime rejects surfaces as the reference's exception text
     {
         bool threw = false;

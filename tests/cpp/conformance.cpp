@@ -222,6 +222,15 @@ static_assert(TransformDPP<>::PAR_ARCH == ParArch::GPU_AMD && defaultParArch == 
 static_assert(exec::pixels_per_thread<float3, float3, false>() == 4 && exec::pixels_per_thread<uchar4, uchar, false>() == 4 &&
               exec::pixels_per_thread<uchar4, float3, false>() == 4 && exec::pixels_per_thread<uchar, uchar, false>() == 16);
 
+// Every public name of the reference's namespace fk (tests/golden/reference_public_names.txt, listed from its headers by
+// tests/golden/make_reference_names.py) exists in this library's fk: a using-declaration of a name that is missing does not
+// compile.  The names that are deliberately absent, each with its reason, are in tests/golden/reference_names_absent.txt.
+namespace reference_names {
+#define FK_REFERENCE_NAME(name) using fk::name;
+#include "reference_names.inc"
+#undef FK_REFERENCE_NAME
+} // namespace reference_names
+
 int main() {
     int failures = 0;
     // RGB2Gray known answers of the reference's unit test (rounding to nearest is not a constant expression)

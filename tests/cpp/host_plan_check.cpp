@@ -1,0 +1,103 @@
+// Host-only check of the launch plans that Executor builds (fk::exec::JobOf::make): no GPU call is made and no device memory
+// is touched; the pointers are made up.  Compiled by hipcc for the host only.
+#include <cstdio>
+#include <vector>
+
+#include "fk/fused_kernel.h"
+
+using namespace fk;
+
+namespace {
+int failures = 0;
+#define CHECK(cond)                                               \
+    do {                                                          \
+        if (!(cond)) {                                            \
+            std::printf("FAILED line %d: %s\n", __LINE__, #cond); \
+            ++failures;                                           \
+        }                                                         \
+    } while (0)
+
+template <typename T>
+RawPtr<ND::_2D, T> image(size_t address, uint w, uint h, uint pitch) {
+    return RawPtr<ND::_2D, T>{ reinterpret_cast<T*>(address), PtrDims<ND::_2D>(w, h, pitch) };
+}
+
+// a three-byte source whose window spans 4 GiB or more must not be addressed with 32-bit offsets: no tile is staged, no
+// line is touched, the taps are read with 64-bit row addresses
+void huge_windows_keep_64_bit_addressing() {
+    const auto write = PerThreadWrite<ND::_2D, float3>::build(image<float3>(0x7000000000ull, 1000, 800, 12000));
+    {
+        const auto read = PerThreadRead<ND::_2D, uchar3>::build(image<uchar3>(0x1000000000ull, 40000, 40000, 120000))
+                              .then(Resize<InterpolationType::INTER_LINEAR>::build(Size(1000, 800)));
+        const auto job = exec::JobOf<std::decay_t<decltype(read)>, std::decay_t<decltype(write)>>::make(read, write);
+        CHECK((job.flags & exec::FLAG_OFFSETS_32) == 0u);
+        CHECK((job.flags & (exec::FLAG_SOURCE_TILE | exec::FLAG_PACKED_TILE)) == 0u);
+        CHECK(job.lds_bytes() == 0u);
+    }
+    {   // up-scaling from a huge source: the tile of float taps would be worth it, and is still refused
+        const auto read = PerThreadRead<ND::_2D, uchar3>::build(image<uchar3>(0x1000000000ull, 40000, 40000, 120000))
+                              .then(Crop<>::build(Rect(10, 10, 500, 39000)))
+                              .then(Resize<InterpolationType::INTER_LINEAR>::build(Size(1000, 800)));
+        const auto job = exec::JobOf<std::decay_t<decltype(read)>, std::decay_t<decltype(write)>>::make(read, write);
+        CHECK((job.flags & exec::FLAG_OFFSETS_32) == 0u);
+        CHECK((job.flags & (exec::FLAG_SOURCE_TILE | exec::FLAG_PACKED_TILE)) == 0u);
+    }
+    {   // the same chains over an ordinary frame take the tiles
+        const auto up = PerThreadRead<ND::_2D, uchar3>::build(image<uchar3>(0x1000000000ull, 3840, 2160, 11520))
+                            .then(Crop<>::build(Rect(0, 0, 500, 400)))
+                            .then(Resize<InterpolationType::INTER_LINEAR>::build(Size(1000, 800)));
+        const auto job = exec::JobOf<std::decay_t<decltype(up)>, std::decay_t<decltype(write)>>::make(up, write);
+        CHECK((job.flags & exec::FLAG_OFFSETS_32) != 0u);
+        CHECK((job.flags & exec::FLAG_SOURCE_TILE) != 0u);
+        const auto down = PerThreadRead<ND::_2D, uchar3>::build(image<uchar3>(0x1000000000ull, 1500, 1200, 4500))
+                              .then(Resize<InterpolationType::INTER_LINEAR>::build(Size(1000, 800)));
+        const auto job2 = exec::JobOf<std::decay_t<decltype(down)>, std::decay_t<decltype(write)>>::make(down, write);
+        CHECK((job2.flags & exec::FLAG_PACKED_TILE) != 0u && job2.lds_bytes() > 0u);
+        // a source that does not start at a whole dword, or whose rows are not whole dwords apart: no packed tile
+        const auto odd = PerThreadRead<ND::_2D, uchar3>::build(image<uchar3>(0x1000000001ull, 1500, 1200, 4500))
+                             .then(Resize<InterpolationType::INTER_LINEAR>::build(Size(1000, 800)));
+        const auto job3 = exec::JobOf<std::decay_t<decltype(odd)>, std::decay_t<decltype(write)>>::make(odd, write);
+        CHECK((job3.flags & exec::FLAG_PACKED_TILE) == 0u);
+        const auto odd_pitch = PerThreadRead<ND::_2D, uchar3>::build(image<uchar3>(0x1000000000ull, 1500, 1200, 4501))
+                                   .then(Resize<InterpolationType::INTER_LINEAR>::build(Size(1000, 800)));
+        const auto job4 = exec::JobOf<std::decay_t<decltype(odd_pitch)>, std::decay_t<decltype(write)>>::make(odd_pitch, write);
+        CHECK((job4.flags & exec::FLAG_PACKED_TILE) == 0u);
+    }
+}
+
+// a batch of windows of different sizes: every plane gets the extent of the batch's thread grid, and the wide (several
+// pixels per thread) path only where the rows below the first are aligned too
+void ragged_batches_take_their_alignment_from_the_whole_box() {
+    // rows 131 bytes apart: a one-row window alone may use the wide path, the same window inside a taller box may not
+    const auto source = image<uchar3>(0x1000000000ull, 41, 60, 131);
+    const auto read = PerThreadRead<ND::_2D, uchar3>::build(source);
+    const auto plane = [&](const Rect& r) { return read.then(Crop<>::build(r)).then(Cast<uchar3, float3>::build()); };
+    using Plane = decltype(plane(Rect()));
+    const std::vector<Plane> planes{ plane(Rect(4, 7, 32, 1)), plane(Rect(0, 0, 16, 9)), plane(Rect(8, 20, 32, 5)) };
+    const auto out = TensorWrite<float3>::build(RawPtr<ND::_3D, float3>{ reinterpret_cast<float3*>(0x7000000000ull), PtrDims<ND::_3D>(36, 12, 3, 1, 36 * 12) });
+    const auto batch = BatchRead<8>::build_first(planes.data(), planes.size());
+    const auto job = exec::JobOf<std::decay_t<decltype(batch)>, std::decay_t<decltype(out)>>::make(batch, out);
+    for (int i = 0; i < 3; ++i) {
+        CHECK(job.plane[i].prog.view.w == 32 && job.plane[i].prog.view.h == 9);
+        CHECK((job.plane[i].flags & exec::FLAG_WHOLE_BOX) != 0u);
+        CHECK((job.plane[i].flags & exec::FLAG_VECTOR_IO) == 0u); // 131-byte rows: no wide accesses below the first row
+    }
+    // alone, the one-row window is not ragged and keeps its own extent
+    const auto single = BatchRead<8>::build_first(planes.data(), 1);
+    const auto job1 = exec::JobOf<std::decay_t<decltype(single)>, std::decay_t<decltype(out)>>::make(single, out);
+    CHECK(job1.plane[0].prog.view.w == 32 && job1.plane[0].prog.view.h == 1 && (job1.plane[0].flags & exec::FLAG_WHOLE_BOX) == 0u);
+    // a part of a larger batch carries the whole batch's box
+    const auto part = BatchRead<8>::build_first(planes.data() + 1, 2, 40, 11);
+    const auto job2 = exec::JobOf<std::decay_t<decltype(part)>, std::decay_t<decltype(out)>>::make(part, out);
+    for (int i = 0; i < 2; ++i) {
+        CHECK(job2.plane[i].prog.view.w == 40 && job2.plane[i].prog.view.h == 11 && (job2.plane[i].flags & exec::FLAG_WHOLE_BOX) != 0u);
+    }
+}
+} // namespace
+
+int main() {
+    huge_windows_keep_64_bit_addressing();
+    ragged_batches_take_their_alignment_from_the_whole_box();
+    if (failures == 0) std::printf("host plans: ok\n");
+    return failures == 0 ? 0 : 1;
+}

@@ -19,6 +19,26 @@ def test_host_api_conformance(native_build):
     assert "conformance ok" in proc.stdout
 
 
+def test_launch_plans_on_the_host(native_build):
+    """Decisions of the host-side plan that no GPU test can reach or see: a three-byte source whose window spans 4 GiB or
+    more keeps 64-bit addressing (no tile, no touch); a ragged batch takes its alignment from the whole box; a batch
+    launched in parts carries the whole batch's box.  No GPU call is made, the pointers are made up."""
+    exe = os.path.join(HERE, "cpp", "host_plan_check")
+    assert os.path.exists(exe), "tests/cpp/host_plan_check is not built (python -m fusedkernellibrary_amd.build)"
+    proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=60)
+    assert proc.returncode == 0 and "host plans: ok" in proc.stdout, proc.stdout
+
+
+def test_staging_ring_state_machine(native_build):
+    """The slots behind fkrt_params_upload / fkrt_params_release with the GPU runtime replaced by stand-ins: a ninth block
+    never overwrites one of eight that are leased, a slot comes back only after its event, the wait for an event does not
+    hold the ring's mutex, twelve host threads never see each other's blocks."""
+    exe = os.path.join(HERE, "cpp", "staging_ring_check")
+    assert os.path.exists(exe), "tests/cpp/staging_ring_check is not built (python -m fusedkernellibrary_amd.build)"
+    proc = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert proc.returncode == 0 and "staging ring: ok" in proc.stdout, proc.stdout
+
+
 @pytest.mark.gpu
 def test_readme_example_as_user_code(oracle, tmp_path):
     exe = os.path.join(HERE, "cpp", "readme_dropin")

@@ -91,6 +91,21 @@ def test_tensor_source(fk, oracle, shape):
     assert same_bits(out.cpu().numpy(), oracle.tensor_mul_f32c3(t, (2.0, -0.5, 1.0001)))
 
 
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 17, 33), (5, 60, 60), (2, 1080, 1920)])
+def test_set_to_fills_every_element_and_nothing_else(fk, shape):
+    """fk::setTo on a float3 tensor: every element receives the value (a fill: the expectation is the value itself), and
+    the elements of a larger allocation around the tensor keep theirs."""
+    planes, h, w = shape
+    around = torch.full((planes * h * w * 3 + 32,), -9.0, device="cuda")
+    out = around[16:-16].view(planes, h, w, 3)
+    fk.set_to_f32c3_tensor((1.5, -2.25, 1e-30), out)
+    torch.cuda.synchronize()
+    got = around.cpu().numpy()
+    want = np.full(got.shape, -9.0, np.float32)
+    want[16:-16] = np.tile(np.array([1.5, -2.25, 1e-30], np.float32), planes * h * w)
+    assert same_bits(got, want)
+
+
 def test_argument_errors_of_these_entry_points(fk, oracle):
     src = dev(oracle.bytes(1, (20, 30, 3)))
     with pytest.raises(fk.FkError, match="1 to 64"):

@@ -33,6 +33,17 @@ def test_no_alloc_entry_point_equals_the_allocating_one(fk, oracle):
         torch.cuda.synchronize()
         assert same_bits(got.cpu().numpy(), want.cpu().numpy()), (len(rects), dst)
         assert same_bits(got.cpu().numpy(), oracle.crop_resize_muls_bgr_tensor(src, rects, dst, *args))
+    # what the entry point exists for: once warmed (the calls above), a call takes no device memory and gives none back
+    rects, dst, aspect = calls[0]
+    args = (aspect, (0.5, 0.25, 0.125), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)
+    got = torch.empty((len(rects), dst[1], dst[0], 3), device="cuda")
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    for _ in range(20):
+        fk.crop_resize_muls_bgr_tensor_noalloc(d, rects, got, *args)
+    free_during = torch.cuda.mem_get_info()[0]
+    torch.cuda.synchronize()
+    assert free_during == free_before and torch.cuda.mem_get_info()[0] == free_before
     with pytest.raises(fk.FkError, match="at most 64 planes"):
         fk.crop_resize_muls_bgr_tensor_noalloc(d, [(0, 0, 8, 8)] * 65, torch.zeros((65, 4, 4, 3), device="cuda"), B.IGNORE_AR, (0,) * 3, (1,) * 3,
                                                (0,) * 3, (1,) * 3)
