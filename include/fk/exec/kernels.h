@@ -1203,6 +1203,7 @@ struct ResizeJob {
                         stride = quads * 4;
                         tile_x0 = 4 * q_lo - s.ox;
                         constexpr int PASSES = 4;
+                        const int wave_of_block = __builtin_amdgcn_readfirstlane(tid >> 6);
                         // item / quads as (item * m) >> 20: exact for every item below N when 2^20 / quads <= m < 2^20 / quads *
                         // (1 + 1 / N).  The reciprocal instruction is within 2^-22 of 1 / quads, so its product with 2^20,
                         // truncated, plus 2 lies between 2^20 / quads + 0.7 and 2^20 / quads + 2.3; with quads <= 64 and fewer
@@ -1223,7 +1224,7 @@ struct ResizeJob {
                             }
 #pragma unroll
                             for (int u = 0; u < PASSES; ++u) {
-                                if (first + BLOCK_THREADS * u < items) { // (uniform: some group of this pass exists)
+                                if (first + BLOCK_THREADS * u + 64 * wave_of_block < items) { // (uniform: some group of this wave's pass exists)
                                     const int wanted = first + BLOCK_THREADS * u + tid;
                                     const int item = wanted < items ? wanted : items - 1;
                                     if constexpr (RAW_SOURCE) {
