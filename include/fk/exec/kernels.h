@@ -838,6 +838,10 @@ struct ResizeJob {
     static_assert(sizeof(Tap) % 4 == 0, "a tap is whole dwords");
     static constexpr int SLOT = static_cast<int>(sizeof(Tap)) / 4; // dwords of a source pixel in the tile
     static constexpr bool READ_IN_PLACE = N > 1;
+    // A short tail is taken into registers once, at the start of the block (read in place it is fetched where it is used, once
+    // per pixel and with the wait in the middle of the arithmetic); a long one is read in place.
+    using Tail = std::decay_t<decltype(Prog::tail)>;
+    using TailHeld = std::conditional_t<(sizeof(Tail) <= 128), Tail, const Tail&>;
     // Three-byte pixels (as they lie in memory, or as the operations fused before the resize leave them, e.g. YUV -> RGB)
     // can also be kept in the tile as one dword each.  Such a tile is filled from aligned pieces of the parent image's
     // rows, four pixels per lane and load, all of a box's loads in flight together; it serves the boxes that the tile of
@@ -975,15 +979,10 @@ struct ResizeJob {
     // (column 0 is window column tile_x0, rows from sy_lo, `stride` dwords per row, only pixels that exist).
     enum : int { TAPS_DIRECT = 0, TAPS_FLOAT_TILE = 1, TAPS_PACKED_TILE = 2 };
     template <int MODE, bool INTERIOR, typename Put>
-    __device__ __attribute__((always_inline)) static inline void sweep(const Prog& prog, const unsigned int* tile, const char* window, const int sx_lo,
+    __device__ __attribute__((always_inline)) static inline void sweep(const View& v, const TailHeld& tail, const unsigned int* tile, const char* window, const int sx_lo,
                                                                       const int sy_lo, const int stride, const int tile_x0, const int x, const int wy0,
                                                                       const int lane, const int wave_rows, const Put& put) {
-        const View& v = prog.view;
         const SrcView& s = v.src;
-        // a short tail is taken into registers once, ahead of the pixels (read in place it is fetched where it is used,
-        // once per pixel and with the wait in the middle of the arithmetic)
-        using Tail = std::decay_t<decltype(prog.tail)>;
-        const std::conditional_t<(sizeof(Tail) <= 128), Tail, const Tail&> tail = prog.tail;
 
         // ---- this lane's column ----
         const int rx = x + v.off_x;
@@ -1136,8 +1135,15 @@ struct ResizeJob {
                 return;
             }
         }
+        // Everything the block needs from the job is read here, in one batch of scalar loads with one wait: the job's own
+        // fields, the plane's view BY VALUE, and the tail.  Read where they are used (through a reference into the kernel
+        // arguments), the same fields arrive one dependent load after the other, ten round trips to the scalar cache between
+        // the start of a block and its first memory request.
         const Prog& prog = job.plane[N == 1 ? 0u : bz];
-        const View& v = prog.view;
+        const View v = prog.view;
+        const TailHeld tail = prog.tail;
+        const unsigned job_flags = job.flags, job_tile_dwords = job.tile_dwords;
+        const Out out = job.out;
         const SrcView& s = v.src;
         const int wave_rows = static_cast<int>(job.wave_rows);
         const int tile_h = (BLOCK_THREADS / 64) * wave_rows;
@@ -1178,7 +1184,7 @@ struct ResizeJob {
             stride = cols | 1;
             const int tile_px = (rx_hi - rx_lo + 1) * (ry_hi - ry_lo + 1);
             // staging pays off while a source pixel is used about once or more; strong down-scaling reads taps directly
-            staged = (job.flags & FLAG_SOURCE_TILE) != 0u && rows * stride * SLOT <= static_cast<int>(job.tile_dwords) && rows * stride * SLOT <= RESIZE_LDS_DWORDS &&
+            staged = (job_flags & FLAG_SOURCE_TILE) != 0u && rows * stride * SLOT <= static_cast<int>(job_tile_dwords) && rows * stride * SLOT <= RESIZE_LDS_DWORDS &&
                      rows * cols <= 3 * tile_px + 256;
             tile_x0 = sx_lo;
             if constexpr (PACKABLE) {
@@ -1191,14 +1197,14 @@ struct ResizeJob {
                 // per source pixel.  Thread t takes groups t, t + 256, ... of the box (rows of `quads` groups); the loads of up
                 // to four of them are issued before the first is used, so a box costs one memory round trip.
                 const int box_px = rows * cols;
-                if (!staged && (job.flags & FLAG_PACKED_TILE) != 0u && box_px <= PACKED_MAX_RATIO * tile_px + 256 &&
+                if (!staged && (job_flags & FLAG_PACKED_TILE) != 0u && box_px <= PACKED_MAX_RATIO * tile_px + 256 &&
                     ((static_cast<unsigned>(reinterpret_cast<size_t>(s.data)) | s.pitch) & 3u) == 0u) {
                     const int last_c = sx_lo + cols - 1 < s.w - 1 ? sx_lo + cols - 1 : s.w - 1; // window columns sx_lo .. last_c
                     const int last_r = sy_lo + rows - 1 < s.h - 1 ? sy_lo + rows - 1 : s.h - 1;
                     const int q_lo = (s.ox + sx_lo) >> 2;
                     const int quads = ((s.ox + last_c) >> 2) - q_lo + 1, box_rows = last_r - sy_lo + 1;
                     const int items = box_rows * quads;
-                    if (quads >= 1 && quads <= 64 && box_rows >= 1 && items * 4 * PSLOT <= static_cast<int>(job.tile_dwords)) {
+                    if (quads >= 1 && quads <= 64 && box_rows >= 1 && items * 4 * PSLOT <= static_cast<int>(job_tile_dwords)) {
                         packed = true;
                         stride = quads * 4;
                         tile_x0 = 4 * q_lo - s.ox;
@@ -1332,7 +1338,7 @@ struct ResizeJob {
                 // (measured: eight 1920x1080 planes to 1280x720 31.3 -> 28.6 us; for larger boxes the touches cost more than
                 // they bring, 3x down-scaling 6.3 -> 7.6 us).
                 const int last_byte = s.w * static_cast<int>(sizeof(Src)) - 4; // last dword that lies wholly inside a window row
-                if (rows * cols <= 3 * tile_px + 256 && last_byte >= 0 && (job.flags & FLAG_OFFSETS_32) != 0u) {
+                if (rows * cols <= 3 * tile_px + 256 && last_byte >= 0 && (job_flags & FLAG_OFFSETS_32) != 0u) {
                     const int row_bytes = cols * static_cast<int>(sizeof(Src));
                     const int first_byte = sx_lo * static_cast<int>(sizeof(Src));
                     const int lines = (row_bytes + 127) / 128 + 1;
@@ -1367,7 +1373,7 @@ struct ResizeJob {
         const auto compute = [&](const auto& put) {
             if (!resamples) {
                 // a tile that lies wholly beside the image (the bars of a preserved aspect ratio): one value for all of it
-                const OutPixel bar = dev::apply_tail(prog.tail, v.background);
+                const OutPixel bar = dev::apply_tail(tail, v.background);
                 for (int g = 0; g < wave_rows; g += RESIZE_GROUP_ROWS) {
                     put(g, std::integral_constant<int, 0>{}, bar);
                     put(g, std::integral_constant<int, 1>{}, bar);
@@ -1375,26 +1381,25 @@ struct ResizeJob {
                     put(g, std::integral_constant<int, 3>{}, bar);
                 }
             } else if (staged) {
-                if (interior) sweep<TAPS_FLOAT_TILE, true>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
-                else sweep<TAPS_FLOAT_TILE, false>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                if (interior) sweep<TAPS_FLOAT_TILE, true>(v, tail, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                else sweep<TAPS_FLOAT_TILE, false>(v, tail, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
             } else if (PACKABLE && packed) {
                 if constexpr (PACKABLE) {
-                    if (interior) sweep<TAPS_PACKED_TILE, true>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
-                    else sweep<TAPS_PACKED_TILE, false>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                    if (interior) sweep<TAPS_PACKED_TILE, true>(v, tail, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                    else sweep<TAPS_PACKED_TILE, false>(v, tail, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
                 }
             } else {
-                if (interior) sweep<TAPS_DIRECT, true>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
-                else sweep<TAPS_DIRECT, false>(prog, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                if (interior) sweep<TAPS_DIRECT, true>(v, tail, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                else sweep<TAPS_DIRECT, false>(v, tail, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
             }
         };
         // One pixel per lane straight from registers: a wave's store covers 64 neighbouring pixels of a row (768
         // consecutive bytes of 12-byte pixels: as fast as 16-byte pieces, measured, and nothing passes through LDS).
-        const Out out = job.out;
         const bool column_here = x < v.w;
         const int rows_here = v.h - wy0; // rows from the wave's first to the plane's last (may exceed the wave's own)
         constexpr bool CAN_STREAM = Out::IS_SPLIT ? sizeof(VBase<OutPixel>) == 4 : (sizeof(OutPixel) % 4 == 0 && sizeof(OutPixel) <= 16);
         if constexpr (CAN_STREAM) {
-            if ((job.flags & FLAG_STREAM_STORES) != 0u) {
+            if ((job_flags & FLAG_STREAM_STORES) != 0u) {
                 // the address of the wave's first row is the same in all its lanes: a descriptor from there on, the row as
                 // the wave's offset (in a scalar register) and the column as the lane's
                 const __amdgpu_buffer_rsrc_t rows = dev::wave_buffer(dev::wave_uniform(
