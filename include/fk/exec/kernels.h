@@ -588,9 +588,8 @@ struct PointwiseJob {
     // A block that lies on one row and owns `span` pixels of it from pixel bx0 on (a whole number of thread groups, so
     // the span is whole 16-byte pieces on both sides).  FULL: span is the block's whole 256*K pixels, nothing is guarded.
     template <bool FULL>
-    __device__ __attribute__((always_inline)) static inline void row_block(const PointwiseJob& job, const Plane& pl, int bx0, int span, int x0, int y,
-                                                                          unsigned bz, int tid, unsigned char* lds) {
-        const View& v = pl.prog.view;
+    __device__ __attribute__((always_inline)) static inline void row_block(const Out& job_out, const Plane& pl, const View& v, const unsigned pl_flags, int bx0, int span,
+                                                                          int x0, int y, unsigned bz, int tid, unsigned char* lds) {
         // A wave's 64 threads own 64*K consecutive pixels, so a wave moves its own span through its own part of the
         // buffer and never waits for the other waves of the block.
         const int wave = tid >> 6, lane = tid & 63;
@@ -636,10 +635,10 @@ struct PointwiseJob {
             }
             dev::wave_sync();
             dev::u32x4* const g = reinterpret_cast<dev::u32x4*>(
-                reinterpret_cast<char*>(job.out.data) + static_cast<size_t>(bz) * job.out.z_stride +
-                static_cast<size_t>(y) * job.out.pitch + static_cast<size_t>(bx0) * sizeof(OutPixel)) + wave * (64 * MINE);
+                reinterpret_cast<char*>(job_out.data) + static_cast<size_t>(bz) * job_out.z_stride +
+                static_cast<size_t>(y) * job_out.pitch + static_cast<size_t>(bx0) * sizeof(OutPixel)) + wave * (64 * MINE);
             const int pieces = span * static_cast<int>(sizeof(OutPixel)) / 16 - wave * (64 * MINE);
-            if ((pl.flags & FLAG_STREAM_STORES) != 0u) {
+            if ((pl_flags & FLAG_STREAM_STORES) != 0u) {
                 // the wave's span starts at the same address for all its lanes
                 const __amdgpu_buffer_rsrc_t span_buffer = dev::wave_buffer(dev::wave_uniform(reinterpret_cast<char*>(g)));
 #pragma unroll
@@ -653,7 +652,7 @@ struct PointwiseJob {
                 }
             }
         } else if (active) {
-            dev::store_group_either<K>((pl.flags & FLAG_STREAM_STORES) != 0u, job.out, x0, y, static_cast<int>(bz), o);
+            dev::store_group_either<K>((pl_flags & FLAG_STREAM_STORES) != 0u, job_out, x0, y, static_cast<int>(bz), o);
         }
     }
 
@@ -666,39 +665,44 @@ struct PointwiseJob {
                 return;
             }
         }
+        // What the block needs from the job, read in one batch of scalar loads (a job that lies in the kernel arguments and is
+        // read through a reference would otherwise fetch each field where it is first used, one dependent round trip after
+        // the other); the tail stays where it is and is read while the pixels are on their way.
         const Plane& pl = job.plane[N == 1 ? 0u : bz];
-        const View& v = pl.prog.view;
+        const View v = pl.prog.view;
+        const unsigned pl_flags = pl.flags, job_grid_x = job.grid_x, job_pair_limit = job.pair_limit, job_tx_shift = job.tx_shift;
+        const Out job_out = job.out;
         const int tid = dev::thread_in_block();
         // pair_limit != 0 (one row per block row, the source shares a chroma row between rows 2k and 2k + 1): workgroups go
         // to the eight XCDs round-robin in launch order, so blocks b and b + 8 run on the same XCD one after the other.
         // Giving them the same columns of rows 2k and 2k + 1 lets the second find the chroma row in that XCD's L2 instead
         // of fetching it from memory again through another one.  The first pair_limit blocks (a multiple of 16 and of two
         // block rows) are dealt out that way among themselves; the few after them keep their places.
-        const unsigned launch_index = bx + job.grid_x * by;
-        if (launch_index < job.pair_limit) {
+        const unsigned launch_index = bx + job_grid_x * by;
+        if (launch_index < job_pair_limit) {
             const unsigned xcd = launch_index & 7u, turn = launch_index >> 3;
             const unsigned pair = 8u * (turn >> 1) + xcd; // (columns, row pair) in the order the XCDs take them up
-            const unsigned k = pair / job.grid_x;
-            bx = pair - k * job.grid_x;
+            const unsigned k = pair / job_grid_x;
+            bx = pair - k * job_grid_x;
             by = 2u * k + (turn & 1u);
         }
-        const int cols = 1 << job.tx_shift;
+        const int cols = 1 << job_tx_shift;
         const int x0 = (static_cast<int>(bx) * cols + (tid & (cols - 1))) * K;
-        const int y = static_cast<int>(by) * (BLOCK_THREADS >> job.tx_shift) + (tid >> job.tx_shift);
+        const int y = static_cast<int>(by) * (BLOCK_THREADS >> job_tx_shift) + (tid >> job_tx_shift);
 
         // FLAG_WHOLE_BOX (a batch of windows of different sizes): every plane produces the extent of the largest, as the
         // reference's thread grid does (batch_operations.h:153-160), so v.w x v.h is that box and elements beside the
         // plane's own window are the parent image's pixels there; where the box leaves the parent image the source pixel
         // is zero.
         bool whole_box = false;
-        if constexpr (std::is_same_v<View, PlainView<Src>>) whole_box = (pl.flags & FLAG_WHOLE_BOX) != 0u;
+        if constexpr (std::is_same_v<View, PlainView<Src>>) whole_box = (pl_flags & FLAG_WHOLE_BOX) != 0u;
         if constexpr (STAGE_IN || STAGE_OUT) {
             // block-uniform decisions
             const int bx0 = static_cast<int>(bx) * BLOCK_THREADS * K; // first pixel of the block
             const int span = v.w - bx0 < BLOCK_THREADS * K ? v.w - bx0 : BLOCK_THREADS * K;
-            if ((pl.flags & FLAG_VECTOR_IO) != 0u && !whole_box && job.tx_shift == 8u && y < v.h && span > 0 && span % K == 0) {
-                if (span == BLOCK_THREADS * K) row_block<true>(job, pl, bx0, span, x0, y, bz, tid, lds);
-                else row_block<false>(job, pl, bx0, span, x0, y, bz, tid, lds);
+            if ((pl_flags & FLAG_VECTOR_IO) != 0u && !whole_box && job_tx_shift == 8u && y < v.h && span > 0 && span % K == 0) {
+                if (span == BLOCK_THREADS * K) row_block<true>(job_out, pl, v, pl_flags, bx0, span, x0, y, bz, tid, lds);
+                else row_block<false>(job_out, pl, v, pl_flags, bx0, span, x0, y, bz, tid, lds);
                 return;
             }
         }
@@ -708,13 +712,13 @@ struct PointwiseJob {
         if constexpr (std::is_same_v<View, PlainView<Src>>) {
             if (whole_box) run_in_parent = v.oy + y < v.img_h && v.ox + x0 + K <= v.img_w;
         }
-        if ((pl.flags & FLAG_VECTOR_IO) != 0u && x0 + K <= v.w && run_in_parent) {
+        if ((pl_flags & FLAG_VECTOR_IO) != 0u && x0 + K <= v.w && run_in_parent) {
             Src in[K];
             Access::template load_group<K>(v, x0, y, in);
             OutPixel o[K];
 #pragma unroll
             for (int k = 0; k < K; ++k) o[k] = dev::apply_tail(pl.prog.tail, in[k]);
-            dev::store_group_either<K>((pl.flags & FLAG_STREAM_STORES) != 0u, job.out, x0, y, static_cast<int>(bz), o);
+            dev::store_group_either<K>((pl_flags & FLAG_STREAM_STORES) != 0u, job_out, x0, y, static_cast<int>(bz), o);
         } else {
             const int xe = x0 + K < v.w ? x0 + K : v.w;
             for (int x = x0; x < xe; ++x) {
@@ -724,7 +728,7 @@ struct PointwiseJob {
                     if (whole_box) in_parent = v.oy + y < v.img_h && v.ox + x < v.img_w;
                 }
                 if (in_parent) pixel = Access::load_one(v, x, y);
-                dev::store_one(job.out, x, y, static_cast<int>(bz), dev::apply_tail(pl.prog.tail, pixel));
+                dev::store_one(job_out, x, y, static_cast<int>(bz), dev::apply_tail(pl.prog.tail, pixel));
             }
         }
     }
@@ -1509,14 +1513,22 @@ struct GenericJob {
     }
 
     // K elements per thread: NEIGHBOURS, or 64 apart (then each of a wave's memory instructions covers 64 neighbours).
+    // the job's own fields as a block holds them (read in one batch at its start; sender and receiver are read in place)
+    struct Held {
+        ActiveThreads active;
+        unsigned stream_rows, packs_rows;
+        char* out_data;
+        unsigned out_pitch;
+        size_t out_z_stride;
+    };
     template <int K, bool NEIGHBOURS>
-    __device__ __attribute__((always_inline)) static inline void body(const GenericJob& job, unsigned bx, unsigned by, unsigned bz) {
+    __device__ __attribute__((always_inline)) static inline void body(const GenericJob& job, const Held& held, unsigned bx, unsigned by, unsigned bz) {
         constexpr int STEP = NEIGHBOURS ? 1 : 64;
         const int tid = dev::thread_in_block();
         const int y = static_cast<int>(by) * 4 + (tid >> 6);
-        const int w = static_cast<int>(job.active.x);
+        const int w = static_cast<int>(held.active.x);
         const int x0 = static_cast<int>(bx) * (64 * K) + (tid & 63) * (NEIGHBOURS ? K : 1);
-        if (x0 >= w || y >= static_cast<int>(job.active.y)) return;
+        if (x0 >= w || y >= static_cast<int>(held.active.y)) return;
         Value value[K];
 #pragma unroll
         for (int k = 0; k < K; ++k) {
@@ -1524,16 +1536,16 @@ struct GenericJob {
             value[k] = Sender::Operation::exec(Point(x, y, static_cast<int>(bz)), job.sender);
         }
         if constexpr (PACKS_ROWS && NEIGHBOURS && K == 4) {
-            if (job.packs_rows != 0u && x0 + K <= w) {
+            if (held.packs_rows != 0u && x0 + K <= w) {
                 constexpr int S = static_cast<int>(sizeof(Value)); // bytes per pixel = dwords per thread
                 unsigned int words[S];
                 dev::pack_pixels<K>(value, words);
-                char* const run = job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch +
+                char* const run = held.out_data + static_cast<size_t>(bz) * held.out_z_stride + static_cast<size_t>(y) * held.out_pitch +
                                   static_cast<size_t>(x0) * S;
-                if (job.stream_rows != 0u) {
+                if (held.stream_rows != 0u) {
                     // the row is the same for the whole wave (a wave is one row of the block)
                     const __amdgpu_buffer_rsrc_t row_buffer = dev::wave_buffer(dev::wave_uniform(
-                        job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch));
+                        held.out_data + static_cast<size_t>(bz) * held.out_z_stride + static_cast<size_t>(y) * held.out_pitch));
                     const unsigned at = static_cast<unsigned>(x0) * S;
                     if constexpr (S == 3) {
                         dev::u32x3 v;
@@ -1550,11 +1562,11 @@ struct GenericJob {
             }
         }
         if constexpr (STREAMS_ROWS) {
-            if (job.stream_rows != 0u) {
+            if (held.stream_rows != 0u) {
                 constexpr int S = static_cast<int>(sizeof(Value));
                 // the row is the same for the whole wave (a wave is one row of the block)
                 const __amdgpu_buffer_rsrc_t row_buffer = dev::wave_buffer(dev::wave_uniform(
-                    job.out_data + static_cast<size_t>(bz) * job.out_z_stride + static_cast<size_t>(y) * job.out_pitch));
+                    held.out_data + static_cast<size_t>(bz) * held.out_z_stride + static_cast<size_t>(y) * held.out_pitch));
 #pragma unroll
                 for (int k = 0; k < K; ++k) {
                     if (x0 + STEP * k < w) {
@@ -1583,15 +1595,17 @@ struct GenericJob {
         }
     }
     __device__ __attribute__((always_inline)) static inline void run(const GenericJob& job, unsigned bx, unsigned by, unsigned bz, unsigned char*) {
-        if (job.xcd_bands != 0u) dev::xcd_band_block(bx, by, bz, job.grid_x, job.grid_y, job.active.z);
+        const Held held{ job.active, job.stream_rows, job.packs_rows, job.out_data, job.out_pitch, job.out_z_stride };
+        const unsigned wide = job.wide, bands = job.xcd_bands, gx = job.grid_x, gy = job.grid_y;
+        if (bands != 0u) dev::xcd_band_block(bx, by, bz, gx, gy, held.active.z);
         if constexpr (PACKS_ROWS) { // the only jobs that are compiled with the neighbour form
-            if (job.wide != 0u && job.packs_rows != 0u) {
-                body<4, true>(job, bx, by, bz);
+            if (wide != 0u && held.packs_rows != 0u) {
+                body<4, true>(job, held, bx, by, bz);
                 return;
             }
         }
-        if (job.wide != 0u) body<4, false>(job, bx, by, bz);
-        else body<1, false>(job, bx, by, bz);
+        if (wide != 0u) body<4, false>(job, held, bx, by, bz);
+        else body<1, false>(job, held, bx, by, bz);
     }
 };
 
@@ -1639,21 +1653,40 @@ template <typename... Jobs>
 struct JobPack;
 template <>
 struct JobPack<> {
-    __device__ __attribute__((always_inline)) static inline void run(const JobPack&, unsigned, unsigned char*) {}
+    static constexpr int COUNT = 0;
+    __device__ __attribute__((always_inline)) static inline void header(const JobPack&, unsigned*, unsigned*, unsigned*) {}
+    template <int I>
+    __device__ __attribute__((always_inline)) static inline void dispatch(const JobPack&, unsigned, const unsigned*, const unsigned*, const unsigned*, unsigned char*) {}
 };
 template <typename Job, typename... Rest>
 struct JobPack<Job, Rest...> {
     Job job;
     unsigned blocks; // blocks of this job: grid_x * grid_y * planes
     JobPack<Rest...> rest;
-    __device__ __attribute__((always_inline)) static inline void run(const JobPack& pack, unsigned block, unsigned char* lds) {
-        if (block < pack.blocks) {
-            const unsigned bx = block % pack.job.grid_x;
-            const unsigned q = block / pack.job.grid_x;
-            Job::run(pack.job, bx, q % pack.job.grid_y, q / pack.job.grid_y, lds);
+    static constexpr int COUNT = 1 + JobPack<Rest...>::COUNT;
+    // The block counts and grids of all the pack's jobs, read in one batch of scalar loads before the block knows which job is
+    // its own (found one job after the other, each count would be a dependent load).
+    __device__ __attribute__((always_inline)) static inline void header(const JobPack& pack, unsigned* blocks_of, unsigned* grid_x_of, unsigned* grid_y_of) {
+        blocks_of[0] = pack.blocks;
+        grid_x_of[0] = pack.job.grid_x;
+        grid_y_of[0] = pack.job.grid_y;
+        JobPack<Rest...>::header(pack.rest, blocks_of + 1, grid_x_of + 1, grid_y_of + 1);
+    }
+    template <int I>
+    __device__ __attribute__((always_inline)) static inline void dispatch(const JobPack& pack, unsigned block, const unsigned* blocks_of, const unsigned* grid_x_of,
+                                                                         const unsigned* grid_y_of, unsigned char* lds) {
+        if (block < blocks_of[I]) {
+            const unsigned bx = block % grid_x_of[I];
+            const unsigned q = block / grid_x_of[I];
+            Job::run(pack.job, bx, q % grid_y_of[I], q / grid_y_of[I], lds);
         } else {
-            JobPack<Rest...>::run(pack.rest, block - pack.blocks, lds);
+            JobPack<Rest...>::template dispatch<I + 1>(pack.rest, block - blocks_of[I], blocks_of, grid_x_of, grid_y_of, lds);
         }
+    }
+    __device__ __attribute__((always_inline)) static inline void run(const JobPack& pack, unsigned block, unsigned char* lds) {
+        unsigned blocks_of[COUNT], grid_x_of[COUNT], grid_y_of[COUNT];
+        header(pack, blocks_of, grid_x_of, grid_y_of);
+        dispatch<0>(pack, block, blocks_of, grid_x_of, grid_y_of, lds);
     }
 };
 template <typename Pack>
