@@ -1286,7 +1286,58 @@ struct ResizeJob {
                 const int block_rows = WAVES * pass_rows;              // rows of a block's pass
                 bool rows_alike = false;
                 if constexpr (RAW_SOURCE && sizeof(Src) == 3) rows_alike = (s.pitch & 3u) == 0u;
-                for (int c = lane & (lane_cols - 1); c < cols; c += lane_cols) {
+                bool staged_by_item = false;
+                if constexpr (RAW_SOURCE && sizeof(Src) == 3) {
+                    if (rows_alike) {
+                        // Three-byte pixels, rows a whole number of dwords apart (the common case): the box's pixels in row-major
+                        // order, thread t takes pixels t, t + 256, ..., the loads of all of them in flight before the first
+                        // is stored, so a box costs one memory round trip with every lane busy (with the lanes
+                        // laid over columns, a box of 35 columns leaves 29 lanes of every wave idle and takes five passes of four
+                        // rows).  item / cols comes from a multiplication by the reciprocal instruction's result: (item + 0.5) / cols
+                        // is at least 0.5 / cols away from a whole number, a tile holds at most 2048 pixels, and the product is off
+                        // by less than 2048 / cols * 2^-21, which is below 0.5 / cols.
+                        staged_by_item = true;
+                        static_assert(RESIZE_LDS_DWORDS / SLOT <= 2048, "the division by multiplication is exact up to 2048 pixels");
+                        const int items = rows * cols;
+                        const float per_col = __builtin_amdgcn_rcpf(static_cast<float>(cols));
+                        const unsigned base = static_cast<unsigned>(reinterpret_cast<size_t>(window));
+                        // (as many passes in flight as the box needs, 2, 4 or 8: a pass that no pixel needs still costs its
+                        // address arithmetic and a repeated load)
+                        const auto stage_passes = [&](const auto passes) {
+                            constexpr int PASSES = decltype(passes)::value;
+                            for (int first = 0; first < items; first += BLOCK_THREADS * PASSES) { // (uniform; one turn for boxes of up to 256 * PASSES pixels)
+                                unsigned int got[PASSES], shift[PASSES];
+                                int at[PASSES];
+#pragma unroll
+                                for (int u = 0; u < PASSES; ++u) {
+                                    const int wanted = first + BLOCK_THREADS * u + tid;
+                                    const int item = wanted < items ? wanted : items - 1;
+                                    const int r = static_cast<int>((static_cast<float>(item) + 0.5f) * per_col);
+                                    const int c = item - r * cols;
+                                    const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
+                                    const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
+                                    const unsigned off = static_cast<unsigned>(sx) * 3u;
+                                    const bool aligned = ((base + off) & 3u) == 0u;
+                                    got[u] = dev::load_dword_from_row(window, static_cast<unsigned>(sy) * s.pitch + off + (aligned ? 1u : 0u));
+                                    shift[u] = aligned ? 0u : 8u;
+                                    at[u] = (r * stride + c) * SLOT;
+                                }
+#pragma unroll
+                                for (int u = 0; u < PASSES; ++u) {
+                                    if (first + BLOCK_THREADS * u + 64 * wave < items) { // (uniform: some pixel of this wave's pass exists)
+                                        dev::PixelSlot<Src> px;
+                                        px.w[0] = got[u] >> shift[u];
+                                        store_tap(tile + at[u], to_tap(dev::slot_to_pixel<Src>(px)));
+                                    }
+                                }
+                            }
+                        };
+                        if (items <= 2 * BLOCK_THREADS) stage_passes(std::integral_constant<int, 2>{});
+                        else if (items <= 4 * BLOCK_THREADS) stage_passes(std::integral_constant<int, 4>{});
+                        else stage_passes(std::integral_constant<int, 8>{});
+                    }
+                }
+                for (int c = lane & (lane_cols - 1); c < cols && !staged_by_item; c += lane_cols) {
                     const int sx = sx_lo + c < s.w - 1 ? sx_lo + c : s.w - 1;
                     // three-byte pixels, rows a whole number of dwords apart: a column has the same alignment in every
                     // row, so a lane's offset and the shift that takes the pixel out of its dword are found once per column
