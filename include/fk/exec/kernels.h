@@ -551,7 +551,7 @@ __device__ __attribute__((always_inline)) inline void fill_default(const Out& ou
 } // namespace dev
 
 // ---- pointwise ---------------------------------------------------------------------------------------------------
-enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_WHOLE_BOX = 8u, FLAG_PACKED_TILE = 16u, FLAG_OFFSETS_32 = 32u };
+enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_WHOLE_BOX = 8u, FLAG_PACKED_TILE = 16u, FLAG_OFFSETS_32 = 32u, FLAG_PAIR_COLUMNS = 64u };
 
 template <typename Prog, size_t N, typename Out, typename Defaults = NoDefaultPlanes>
 struct PointwiseJob {
@@ -1150,6 +1150,15 @@ struct ResizeJob {
         const Out out = job.out;
         const SrcView& s = v.src;
         const int wave_rows = static_cast<int>(job.wave_rows);
+        // FLAG_PAIR_COLUMNS: workgroups reach the eight XCDs round-robin in launch order, and each XCD has an L2 of its own.  Two
+        // tiles that are neighbours along x read the same cache lines where their source boxes meet (a tile's row of source
+        // pixels is often shorter than a line), so within every run of sixteen tile columns the blocks are dealt out such that
+        // launch positions p and p + 8, which run on the same XCD at the same time, work on columns 2p and 2p + 1: the second
+        // request for a shared line is served by that XCD's L2.
+        if ((job_flags & FLAG_PAIR_COLUMNS) != 0u && bx < (job.grid_x & ~15u)) {
+            const unsigned p = bx & 15u;
+            bx = (bx & ~15u) + 2u * (p & 7u) + (p >> 3);
+        }
         const int tile_h = (BLOCK_THREADS / 64) * wave_rows;
         const int tx0 = static_cast<int>(bx) * RESIZE_TILE_W;
         const int ty0 = static_cast<int>(by) * tile_h;
