@@ -184,7 +184,11 @@ struct JobOf {
                 // tile height, grid rows and LDS layout; sets FLAG_SOURCE_TILE when some plane's tiles are worth staging
                 job.grid_y = job.plan(used, max_h, resize_wave_rows_override(), resize_packed_capacity());
                 // x-neighbouring tiles in pairs on one XCD (FK_RESIZE_NO_PAIRS switches it off: for measurements)
-                if (job.grid_x >= 16u && std::getenv("FK_RESIZE_NO_PAIRS") == nullptr) job.flags |= FLAG_PAIR_COLUMNS;
+                if (std::getenv("FK_RESIZE_NO_PAIRS") == nullptr) {
+                    const unsigned gx = job.grid_x;
+                    if (gx > 9u) job.flags |= FLAG_PAIR_COLUMNS;
+                    else if (gx > 1u && (gx & (gx - 1u)) == 0u && gx * job.grid_y > 9u) job.flags |= FLAG_PAIR_TILES;
+                }
                 return job;
             } else {
                 using Job = PointwiseJob<Prog, N, Out, Defaults>;

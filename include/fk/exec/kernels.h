@@ -542,6 +542,22 @@ struct NoDefaultPlanes {
     static constexpr bool ENABLED = false;
 };
 namespace dev {
+// Launch position l of n -> an index of 0 .. n-1 (a permutation) such that positions 8 apart, which run on the same XCD,
+// get the indices 2k and 2k + 1: whole runs of sixteen positions are dealt out as eight such pairs, and a last run of
+// more than eight positions as the pairs it has, followed by what is left.
+__host__ __device__ __attribute__((always_inline)) inline unsigned deal_pairs(const unsigned l, const unsigned n) {
+    const unsigned whole = n & ~15u;
+    if (l < whole) {
+        const unsigned p = l & 15u;
+        return (l & ~15u) + 2u * (p & 7u) + (p >> 3);
+    }
+    const unsigned last = n - whole, k = l - whole;
+    if (last <= 8u) return l;
+    const unsigned pairs = last - 8u;
+    if (k < pairs) return whole + 2u * k;
+    if (k >= 8u) return whole + 2u * (k - 8u) + 1u;
+    return l + pairs;
+}
 // the part of such a plane that lies in columns x0 .. x0 + nx - 1 of row y, written by one thread
 template <typename Out, typename O>
 __device__ __attribute__((always_inline)) inline void fill_default(const Out& out, const DefaultPlanes<O>& d, int x0, int nx, int y, int z) {
@@ -551,7 +567,7 @@ __device__ __attribute__((always_inline)) inline void fill_default(const Out& ou
 } // namespace dev
 
 // ---- pointwise ---------------------------------------------------------------------------------------------------
-enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_WHOLE_BOX = 8u, FLAG_PACKED_TILE = 16u, FLAG_OFFSETS_32 = 32u, FLAG_PAIR_COLUMNS = 64u };
+enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_WHOLE_BOX = 8u, FLAG_PACKED_TILE = 16u, FLAG_OFFSETS_32 = 32u, FLAG_PAIR_COLUMNS = 64u, FLAG_PAIR_TILES = 128u };
 
 template <typename Prog, size_t N, typename Out, typename Defaults = NoDefaultPlanes>
 struct PointwiseJob {
@@ -1150,14 +1166,19 @@ struct ResizeJob {
         const Out out = job.out;
         const SrcView& s = v.src;
         const int wave_rows = static_cast<int>(job.wave_rows);
-        // FLAG_PAIR_COLUMNS: workgroups reach the eight XCDs round-robin in launch order, and each XCD has an L2 of its own.  Two
-        // tiles that are neighbours along x read the same cache lines where their source boxes meet (a tile's row of source
-        // pixels is often shorter than a line), so within every run of sixteen tile columns the blocks are dealt out such that
-        // launch positions p and p + 8, which run on the same XCD at the same time, work on columns 2p and 2p + 1: the second
-        // request for a shared line is served by that XCD's L2.
-        if ((job_flags & FLAG_PAIR_COLUMNS) != 0u && bx < (job.grid_x & ~15u)) {
-            const unsigned p = bx & 15u;
-            bx = (bx & ~15u) + 2u * (p & 7u) + (p >> 3);
+        // FLAG_PAIR_COLUMNS / FLAG_PAIR_TILES: workgroups reach the eight XCDs round-robin in launch order, and each XCD has an
+        // L2 of its own.  Two tiles that are neighbours along x read the same cache lines where their source boxes meet (a
+        // tile's row of source pixels is often shorter than a line), so the blocks of a row of tiles (of a whole plane, when
+        // its rows are a power of two of at most eight tiles) are dealt out such that launch positions p and p + 8, which
+        // run on the same XCD at the same time, work on columns 2k and 2k + 1: the second request for a shared line is
+        // served by that XCD's L2.
+        if ((job_flags & FLAG_PAIR_COLUMNS) != 0u) {
+            bx = dev::deal_pairs(bx, job.grid_x);
+        } else if ((job_flags & FLAG_PAIR_TILES) != 0u) {
+            const unsigned gx = job.grid_x, shift = 31u - static_cast<unsigned>(__builtin_clz(gx));
+            const unsigned t = dev::deal_pairs(bx + (by << shift), gx * job.grid_y);
+            bx = t & (gx - 1u);
+            by = t >> shift;
         }
         const int tile_h = (BLOCK_THREADS / 64) * wave_rows;
         const int tx0 = static_cast<int>(bx) * RESIZE_TILE_W;

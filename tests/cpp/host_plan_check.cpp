@@ -93,10 +93,28 @@ void ragged_batches_take_their_alignment_from_the_whole_box() {
         CHECK(job2.plane[i].prog.view.w == 40 && job2.plane[i].prog.view.h == 11 && (job2.plane[i].flags & exec::FLAG_WHOLE_BOX) != 0u);
     }
 }
+
+// The dealing of tiles to launch positions is a permutation for every count, and puts the tiles 2k and 2k + 1 on launch
+// positions that are 8 apart (the same XCD) wherever the count leaves room for it.
+void tile_pairs_are_a_permutation_with_neighbours_eight_apart() {
+    for (unsigned n = 1; n < 300; ++n) {
+        std::vector<int> position(n, -1);
+        for (unsigned l = 0; l < n; ++l) {
+            const unsigned t = exec::dev::deal_pairs(l, n);
+            CHECK(t < n && position[t < n ? t : 0] < 0);
+            if (t < n) position[t] = static_cast<int>(l);
+        }
+        unsigned together = 0;
+        for (unsigned t = 0; t + 1 < n; t += 2) together += (position[t + 1] - position[t] == 8) ? 1u : 0u;
+        const unsigned last = n & 15u;
+        CHECK(together == (n >> 4) * 8u + (last > 8u ? last - 8u : 0u));
+    }
+}
 } // namespace
 
 int main() {
     huge_windows_keep_64_bit_addressing();
+    tile_pairs_are_a_permutation_with_neighbours_eight_apart();
     ragged_batches_take_their_alignment_from_the_whole_box();
     if (failures == 0) std::printf("host plans: ok\n");
     return failures == 0 ? 0 : 1;
