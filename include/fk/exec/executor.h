@@ -184,6 +184,8 @@ struct JobOf {
                 // tile height, grid rows and LDS layout; sets FLAG_SOURCE_TILE when some plane's tiles are worth staging
                 job.grid_y = job.plan(used, max_h, resize_wave_rows_override(), resize_packed_capacity());
                 // x-neighbouring tiles in pairs on one XCD (FK_RESIZE_NO_PAIRS switches it off: for measurements)
+                if (std::getenv("FK_RESIZE_NO_QUAD_FILL") != nullptr) job.flags &= ~FLAG_QUAD_FILL; // (for measurements)
+                if (const char* pad = std::getenv("FK_RESIZE_LDS_DWORDS")) { if (job.tile_dwords != 0u) { const unsigned want = static_cast<unsigned>(std::strtoul(pad, nullptr, 10)); job.tile_dwords = want > job.tile_dwords ? want : job.tile_dwords; } }
                 if (std::getenv("FK_RESIZE_NO_PAIRS") == nullptr) {
                     const unsigned gx = job.grid_x;
                     if (gx > 9u) job.flags |= FLAG_PAIR_COLUMNS;

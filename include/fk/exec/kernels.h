@@ -407,11 +407,14 @@ struct SourceAccess<PlainView<T>> {
         px[2] = __builtin_amdgcn_alignbyte(w.z, w.y, 2u);
         px[3] = w.z >> 8u;
     }
+    // the four pixels as their type, each channel taken from the byte of the dword that holds it (a conversion to float
+    // that follows is then one instruction per channel)
     __device__ __attribute__((always_inline)) static inline void quad_pixels(const Quad& w, T* px) {
-        unsigned int d[4];
-        quad_dwords(w, d);
+        using B = VBase<T>;
+        const unsigned int d[3] = { w.x, w.y, w.z };
+        const auto channel = [&](const int byte) { return static_cast<B>(static_cast<unsigned char>(d[byte >> 2] >> (8 * (byte & 3)))); };
 #pragma unroll
-        for (int k = 0; k < 4; ++k) px[k] = dev::unpack3<T>(d[k]);
+        for (int k = 0; k < 4; ++k) px[k] = T{ channel(3 * k), channel(3 * k + 1), channel(3 * k + 2) };
     }
 };
 
@@ -567,7 +570,7 @@ __device__ __attribute__((always_inline)) inline void fill_default(const Out& ou
 } // namespace dev
 
 // ---- pointwise ---------------------------------------------------------------------------------------------------
-enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_WHOLE_BOX = 8u, FLAG_PACKED_TILE = 16u, FLAG_OFFSETS_32 = 32u, FLAG_PAIR_COLUMNS = 64u, FLAG_PAIR_TILES = 128u };
+enum : unsigned { FLAG_VECTOR_IO = 1u, FLAG_STREAM_STORES = 2u, FLAG_SOURCE_TILE = 4u, FLAG_WHOLE_BOX = 8u, FLAG_PACKED_TILE = 16u, FLAG_OFFSETS_32 = 32u, FLAG_PAIR_COLUMNS = 64u, FLAG_PAIR_TILES = 128u, FLAG_QUAD_FILL = 256u };
 
 template <typename Prog, size_t N, typename Out, typename Defaults = NoDefaultPlanes>
 struct PointwiseJob {
@@ -902,6 +905,16 @@ struct ResizeJob {
         const bool worth = rows * (cols | 1) * SLOT <= RESIZE_LDS_DWORDS && rows * cols <= 3 * RESIZE_TILE_W * tile_h + 256;
         return worth ? static_cast<unsigned>(rows * (cols | 1) * SLOT) : 0u;
     }
+    // dwords of a tile of float taps that is filled from aligned groups of four pixels (an upper bound of what any tile of
+    // a plane with these factors needs), 0 when the plane's tiles are not worth float taps or too wide for it: a row of the
+    // tile holds the groups that cover the box's columns and one group more, for the copy of the window's last column
+    static unsigned quad_filled_tile_dwords(float fx, float fy, int tile_h) {
+        if (staged_tile_dwords(fx, fy, tile_h) == 0u) return 0u;
+        const int cols = static_cast<int>((RESIZE_TILE_W - 1) * fx) + 3, rows = static_cast<int>((tile_h - 1) * fy) + 3;
+        const int quads = (cols + 6) / 4;
+        const unsigned need = static_cast<unsigned>(rows * 4 * (quads + 1) * SLOT);
+        return quads <= 64 && need <= static_cast<unsigned>(RESIZE_PACKED_DWORDS) ? need : 0u;
+    }
     // whether the byte offset of every pixel of a window, from the window's first pixel, fits 32 bits (with room for the
     // few bytes that an access adds)
     static bool window_fits_32_bits(const SrcView& s) {
@@ -953,6 +966,13 @@ struct ResizeJob {
             const unsigned need = staged_tile_dwords(plane[i].view.fx, plane[i].view.fy, tile_h());
             if (need != 0u) flags |= FLAG_SOURCE_TILE;
             tile_dwords = need > tile_dwords ? need : tile_dwords;
+            if constexpr (PACKABLE && RAW_SOURCE) {
+                if (need != 0u && packable && Access::quads_aligned(plane[i].view.src)) {
+                    const unsigned filled = quad_filled_tile_dwords(plane[i].view.fx, plane[i].view.fy, tile_h());
+                    if (filled != 0u) flags |= FLAG_QUAD_FILL;
+                    tile_dwords = filled > tile_dwords ? filled : tile_dwords;
+                }
+            }
             if constexpr (PACKABLE) {
                 if (need == 0u && packable && Access::quads_aligned(plane[i].view.src)) {
                     const unsigned packed = packed_tile_dwords(plane[i].view.fx, plane[i].view.fy, tile_h(), packed_capacity);
@@ -1317,8 +1337,75 @@ struct ResizeJob {
                 bool rows_alike = false;
                 if constexpr (RAW_SOURCE && sizeof(Src) == 3) rows_alike = (s.pitch & 3u) == 0u;
                 bool staged_by_item = false;
+                if constexpr (RAW_SOURCE && PACKABLE) {
+                    // Three-byte pixels of an image that starts at a whole dword, rows a whole number of dwords apart: the tile
+                    // is filled from the aligned groups of four pixels (twelve bytes, one load) that cover the box's columns,
+                    // read through a descriptor of the whole parent image, so a thread converts four pixels per load and
+                    // address instead of one.  The tile's column 0 is the first group's first pixel, a row holds the groups and
+                    // room for one more; rows past the window's last are the last one again, and where the box reaches past
+                    // the window's last column, that column's copy is written behind it once the groups are in place.
+                    if ((job_flags & FLAG_QUAD_FILL) != 0u && ((static_cast<unsigned>(reinterpret_cast<size_t>(s.data)) | s.pitch) & 3u) == 0u) {
+                        const int last_c = sx_lo + cols - 1 < s.w - 1 ? sx_lo + cols - 1 : s.w - 1;
+                        const int q_lo = (s.ox + sx_lo) >> 2;
+                        const int quads = ((s.ox + last_c) >> 2) - q_lo + 1;
+                        const int row_px = 4 * (quads + 1);
+                        const int items = rows * quads;
+                        const int behind = sx_lo + cols - 1 - last_c; // columns of the box behind the window's last (0 or 1)
+                        if (quads >= 1 && quads <= 64 && behind <= 3 && rows * row_px * SLOT <= static_cast<int>(job_tile_dwords)) {
+                            staged_by_item = true;
+                            stride = row_px;
+                            tile_x0 = 4 * q_lo - s.ox;
+                            constexpr int PASSES = 2;
+                            // (item / quads as (item * m) >> 20: see the tiles of packed pixels above; a tile of float taps holds
+                            // fewer groups than one of packed pixels)
+                            const unsigned m = static_cast<unsigned>(1048576.0f * __builtin_amdgcn_rcpf(static_cast<float>(quads))) + 2u;
+                            const __amdgpu_buffer_rsrc_t image = Access::quad_buffer(s);
+                            for (int first = 0; first < items; first += BLOCK_THREADS * PASSES) { // (uniform)
+                                typename Access::Quad raw[PASSES];
+                                int at[PASSES];
+#pragma unroll
+                                for (int u = 0; u < PASSES; ++u) {
+                                    const int wanted = first + BLOCK_THREADS * u + tid;
+                                    const int item = wanted < items ? wanted : items - 1;
+                                    const int r = static_cast<int>((static_cast<unsigned>(item) * m) >> 20);
+                                    const int q = item - r * quads;
+                                    const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
+                                    raw[u] = Access::load_quad(image, s, q_lo + q, s.oy + sy);
+                                    at[u] = (r * row_px + 4 * q) * SLOT;
+                                }
+#pragma unroll
+                                for (int u = 0; u < PASSES; ++u) {
+                                    if (first + BLOCK_THREADS * u + 64 * wave < items) { // (uniform: some group of this wave's pass exists)
+                                        Src px[4];
+                                        Access::quad_pixels(raw[u], px);
+                                        unsigned int taps[4 * SLOT];
+#pragma unroll
+                                        for (int k = 0; k < 4; ++k) {
+                                            const Tap t = to_tap(px[k]);
+                                            __builtin_memcpy(taps + k * SLOT, &t, sizeof(Tap));
+                                        }
+#pragma unroll
+                                        for (int k = 0; k < SLOT; ++k) {
+                                            dev::u32x4 piece;
+                                            piece.x = taps[4 * k]; piece.y = taps[4 * k + 1]; piece.z = taps[4 * k + 2]; piece.w = taps[4 * k + 3];
+                                            reinterpret_cast<dev::u32x4*>(tile + at[u])[k] = piece;
+                                        }
+                                    }
+                                }
+                            }
+                            if (behind > 0) { // (uniform) the box wants the column behind the window's last
+                                dev::block_sync();
+                                const int copy = s.w - tile_x0;
+                                for (int r = tid; r < rows; r += BLOCK_THREADS) {
+                                    const Tap edge = load_tap(tile + (r * row_px + copy - 1) * SLOT);
+                                    for (int j = 0; j < behind; ++j) store_tap(tile + (r * row_px + copy + j) * SLOT, edge);
+                                }
+                            }
+                        }
+                    }
+                }
                 if constexpr (RAW_SOURCE && sizeof(Src) == 3) {
-                    if (rows_alike) {
+                    if (rows_alike && !staged_by_item) {
                         // Three-byte pixels, rows a whole number of dwords apart (the common case): the box's pixels in row-major
                         // order, thread t takes pixels t, t + 256, ..., the loads of all of them in flight before the first
                         // is stored, so a box costs one memory round trip with every lane busy (with the lanes
@@ -1466,8 +1553,9 @@ struct ResizeJob {
                     put(g, std::integral_constant<int, 3>{}, bar);
                 }
             } else if (staged) {
-                if (interior) sweep<TAPS_FLOAT_TILE, true>(v, tail, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
-                else sweep<TAPS_FLOAT_TILE, false>(v, tail, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                // (the tile's column 0 is window column tile_x0: the box's first column, or the first pixel of the group that holds it)
+                if (interior) sweep<TAPS_FLOAT_TILE, true>(v, tail, tile, window, tile_x0, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
+                else sweep<TAPS_FLOAT_TILE, false>(v, tail, tile, window, tile_x0, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
             } else if (PACKABLE && packed) {
                 if constexpr (PACKABLE) {
                     if (interior) sweep<TAPS_PACKED_TILE, true>(v, tail, tile, window, sx_lo, sy_lo, stride, tile_x0, x, wy0, lane, wave_rows, put);
