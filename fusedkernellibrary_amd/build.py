@@ -93,10 +93,15 @@ def build_cpp_tests():
 
 
 def build_benchmarks():
-    """benchmarks/reference_sweeps: the reference's four benchmark sweeps as user code of the operator API."""
+    """benchmarks/reference_sweeps: the reference's four benchmark sweeps as user code of the operator API; and
+    benchmarks/store_patterns."""
     src = os.path.join(HERE, "benchmarks", "reference_sweeps.cpp")
     out = os.path.join(HERE, "benchmarks", "reference_sweeps")
     _run([hipcc(), "-x", "hip", src, "-I" + INCLUDE, *DEVICE_FLAGS, "-L" + HERE, "-lfk_hip_rt", "-Wl,-rpath,$ORIGIN/..", "-o", out])
+    # benchmarks/store_patterns: what the headline's output costs to write, by store pattern (a program of its own against the
+    # HIP runtime; it uses nothing of the library)
+    _run([hipcc(), os.path.join(HERE, "benchmarks", "store_patterns.hip"), "--offload-arch=gfx950", "-O3", "-Wno-unused-value",
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", os.path.join(HERE, "benchmarks", "store_patterns")])
     return out
 
 
