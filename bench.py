@@ -85,8 +85,8 @@ def percentile(sorted_values, q):
 
 def time_blocks(timer, launch, steps, warmup, blocks):
     """`blocks` timed blocks of exactly `steps` launches each, every block bracketed by a device synchronisation on both
-    sides: per block the wall time per step and the time per launch by HIP events on the launch stream.  Returns the two
-    lists (milliseconds per step), in the order measured."""
+    sides: per block the wall time per step and the time per launch by HIP events on the launch stream (over the block's
+    launches but the first).  Returns the two lists (milliseconds per step), in the order measured."""
     import torch
     spin_up(launch)
     for i in range(warmup):
@@ -104,13 +104,23 @@ def time_blocks(timer, launch, steps, warmup, blocks):
                 launch(i)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        timer.start()
-        for i in range(steps):
-            launch(n + i)
-        ev = timer.stop_ms()
+        # The wall clock covers all `steps` launches.  The event pair covers all but the first: the device is idle when the
+        # block starts, so between an event recorded first and the first kernel lies the host's time to issue that launch
+        # (10-20 us, which a block of 20 launches would spread over its kernels as a microsecond each).  Recorded behind the
+        # first launch, the opening event completes when that kernel ends, and the others follow it back to back.
+        if steps > 1:
+            launch(n)
+            timer.start()
+            for i in range(1, steps):
+                launch(n + i)
+            ev = timer.stop_ms() / (steps - 1)
+        else:
+            timer.start()
+            launch(n)
+            ev = timer.stop_ms()
         torch.cuda.synchronize()
         wall.append((time.perf_counter() - t0) * 1e3 / steps)
-        events.append(ev / steps)
+        events.append(ev)
         n += steps
     return wall, events
 

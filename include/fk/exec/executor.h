@@ -72,6 +72,21 @@ inline unsigned resize_packed_capacity() {
     return dwords;
 }
 
+// Switches for measurements, read once: FK_RESIZE_NO_QUAD_FILL (tiles of float taps filled one pixel per thread),
+// FK_RESIZE_NO_PAIRS (tiles in launch order), FK_RESIZE_LDS_DWORDS=n (a launch that uses LDS asks for at least n dwords per block).
+struct ResizeSwitches {
+    bool no_quad_fill, no_pairs;
+    unsigned lds_dwords;
+};
+inline const ResizeSwitches& resize_switches() {
+    static const ResizeSwitches switches = [] {
+        const char* lds = std::getenv("FK_RESIZE_LDS_DWORDS");
+        return ResizeSwitches{ std::getenv("FK_RESIZE_NO_QUAD_FILL") != nullptr, std::getenv("FK_RESIZE_NO_PAIRS") != nullptr,
+                               lds != nullptr ? static_cast<unsigned>(std::strtoul(lds, nullptr, 10)) : 0u };
+    }();
+    return switches;
+}
+
 // ---- job construction ----------------------------------------------------------------------------------------
 namespace detail {
 // operations that resample through a matrix (Warping): their taps wander over the source rows
@@ -184,9 +199,10 @@ struct JobOf {
                 // tile height, grid rows and LDS layout; sets FLAG_SOURCE_TILE when some plane's tiles are worth staging
                 job.grid_y = job.plan(used, max_h, resize_wave_rows_override(), resize_packed_capacity());
                 // x-neighbouring tiles in pairs on one XCD (FK_RESIZE_NO_PAIRS switches it off: for measurements)
-                if (std::getenv("FK_RESIZE_NO_QUAD_FILL") != nullptr) job.flags &= ~FLAG_QUAD_FILL; // (for measurements)
-                if (const char* pad = std::getenv("FK_RESIZE_LDS_DWORDS")) { if (job.tile_dwords != 0u) { const unsigned want = static_cast<unsigned>(std::strtoul(pad, nullptr, 10)); job.tile_dwords = want > job.tile_dwords ? want : job.tile_dwords; } }
-                if (std::getenv("FK_RESIZE_NO_PAIRS") == nullptr) {
+                const ResizeSwitches& switches = resize_switches();
+                if (switches.no_quad_fill) job.flags &= ~FLAG_QUAD_FILL;
+                if (job.tile_dwords != 0u && switches.lds_dwords > job.tile_dwords) job.tile_dwords = switches.lds_dwords;
+                if (!switches.no_pairs) {
                     const unsigned gx = job.grid_x;
                     if (gx > 9u) job.flags |= FLAG_PAIR_COLUMNS;
                     else if (gx > 1u && (gx & (gx - 1u)) == 0u && gx * job.grid_y > 9u) job.flags |= FLAG_PAIR_TILES;
