@@ -913,7 +913,9 @@ struct ResizeJob {
         const int cols = static_cast<int>((RESIZE_TILE_W - 1) * fx) + 3, rows = static_cast<int>((tile_h - 1) * fy) + 3;
         const int quads = (cols + 6) / 4;
         const unsigned need = static_cast<unsigned>(rows * 4 * (quads + 1) * SLOT);
-        return quads <= 64 && need <= static_cast<unsigned>(RESIZE_PACKED_DWORDS) ? need : 0u;
+        // (one group per thread: boxes that need two per thread are filled no faster this way than one pixel per thread, the
+        // headline's 47 x 25 boxes 23.2-24.3 against 23.1 us by box of the pool)
+        return rows * quads <= BLOCK_THREADS && need <= static_cast<unsigned>(RESIZE_PACKED_DWORDS) ? need : 0u;
     }
     // whether the byte offset of every pixel of a window, from the window's first pixel, fits 32 bits (with room for the
     // few bytes that an access adds)
@@ -967,7 +969,9 @@ struct ResizeJob {
             if (need != 0u) flags |= FLAG_SOURCE_TILE;
             tile_dwords = need > tile_dwords ? need : tile_dwords;
             if constexpr (PACKABLE && RAW_SOURCE) {
-                if (need != 0u && packable && Access::quads_aligned(plane[i].view.src)) {
+                // (launches of 64 x 16 tiles keep the fill of one pixel per thread: the 50-crop batch took 13.35 us this way
+                // against 13.05 us, the 16:9 crops in 64 x 32 tiles 22.9 against 23.5 us)
+                if (need != 0u && wave_rows >= 8u && packable && Access::quads_aligned(plane[i].view.src)) {
                     const unsigned filled = quad_filled_tile_dwords(plane[i].view.fx, plane[i].view.fy, tile_h());
                     if (filled != 0u) flags |= FLAG_QUAD_FILL;
                     tile_dwords = filled > tile_dwords ? filled : tile_dwords;
@@ -1343,7 +1347,7 @@ struct ResizeJob {
                     // read through a descriptor of the whole parent image, so a thread converts four pixels per load and
                     // address instead of one.  The tile's column 0 is the first group's first pixel, a row holds the groups and
                     // room for one more; rows past the window's last are the last one again, and where the box reaches past
-                    // the window's last column, that column's copy is written behind it once the groups are in place.
+                    // the window's last column, the thread that fetched that column writes its copy behind it.
                     if ((job_flags & FLAG_QUAD_FILL) != 0u && ((static_cast<unsigned>(reinterpret_cast<size_t>(s.data)) | s.pitch) & 3u) == 0u) {
                         const int last_c = sx_lo + cols - 1 < s.w - 1 ? sx_lo + cols - 1 : s.w - 1;
                         const int q_lo = (s.ox + sx_lo) >> 2;
@@ -1351,18 +1355,23 @@ struct ResizeJob {
                         const int row_px = 4 * (quads + 1);
                         const int items = rows * quads;
                         const int behind = sx_lo + cols - 1 - last_c; // columns of the box behind the window's last (0 or 1)
-                        if (quads >= 1 && quads <= 64 && behind <= 3 && rows * row_px * SLOT <= static_cast<int>(job_tile_dwords)) {
+                        // (boxes of up to one group per thread, as the host planned for the plane's factors)
+                        if (quads >= 1 && items <= BLOCK_THREADS && behind <= 3 && rows * row_px * SLOT <= static_cast<int>(job_tile_dwords)) {
                             staged_by_item = true;
                             stride = row_px;
                             tile_x0 = 4 * q_lo - s.ox;
-                            constexpr int PASSES = 2;
                             // (item / quads as (item * m) >> 20: see the tiles of packed pixels above; a tile of float taps holds
                             // fewer groups than one of packed pixels)
                             const unsigned m = static_cast<unsigned>(1048576.0f * __builtin_amdgcn_rcpf(static_cast<float>(quads))) + 2u;
                             const __amdgpu_buffer_rsrc_t image = Access::quad_buffer(s);
-                            for (int first = 0; first < items; first += BLOCK_THREADS * PASSES) { // (uniform)
+                            // the window's last column inside its group, and where its copies go from the start of that group
+                            const int edge_pixel = (s.ox + s.w - 1) & 3;
+                            const int edge_slot = (s.w - tile_x0 - 4 * (quads - 1)) * SLOT;
+                            constexpr int PASSES = 1;
+                            for (int first = 0; first < items; first += BLOCK_THREADS * PASSES) { // (uniform: one turn)
                                 typename Access::Quad raw[PASSES];
                                 int at[PASSES];
+                                bool last_group[PASSES];
 #pragma unroll
                                 for (int u = 0; u < PASSES; ++u) {
                                     const int wanted = first + BLOCK_THREADS * u + tid;
@@ -1372,6 +1381,7 @@ struct ResizeJob {
                                     const int sy = sy_lo + r < s.h - 1 ? sy_lo + r : s.h - 1;
                                     raw[u] = Access::load_quad(image, s, q_lo + q, s.oy + sy);
                                     at[u] = (r * row_px + 4 * q) * SLOT;
+                                    last_group[u] = q == quads - 1;
                                 }
 #pragma unroll
                                 for (int u = 0; u < PASSES; ++u) {
@@ -1390,15 +1400,19 @@ struct ResizeJob {
                                             piece.x = taps[4 * k]; piece.y = taps[4 * k + 1]; piece.z = taps[4 * k + 2]; piece.w = taps[4 * k + 3];
                                             reinterpret_cast<dev::u32x4*>(tile + at[u])[k] = piece;
                                         }
+                                        // The copies of the window's last column behind it, by the thread that holds that column (its
+                                        // row's last group), after its own stores: the copy lies inside that group or in the room
+                                        // behind it, which no other thread writes.
+                                        if (behind > 0) { // (uniform)
+                                            Src edge = px[0];
+                                            if (edge_pixel == 1) edge = px[1];
+                                            if (edge_pixel == 2) edge = px[2];
+                                            if (edge_pixel == 3) edge = px[3];
+                                            if (last_group[u]) {
+                                                for (int j = 0; j < behind; ++j) store_tap(tile + at[u] + edge_slot + j * SLOT, to_tap(edge));
+                                            }
+                                        }
                                     }
-                                }
-                            }
-                            if (behind > 0) { // (uniform) the box wants the column behind the window's last
-                                dev::block_sync();
-                                const int copy = s.w - tile_x0;
-                                for (int r = tid; r < rows; r += BLOCK_THREADS) {
-                                    const Tap edge = load_tap(tile + (r * row_px + copy - 1) * SLOT);
-                                    for (int j = 0; j < behind; ++j) store_tap(tile + (r * row_px + copy + j) * SLOT, edge);
                                 }
                             }
                         }
