@@ -65,6 +65,29 @@ void huge_windows_keep_64_bit_addressing() {
     }
 }
 
+// which launches fill their tiles of float taps from aligned groups of four pixels: three-byte images with dword-aligned
+// rows, 64 x 32 tiles (launches of 1024 tiles and more), boxes of at most one group per thread
+void tiles_are_filled_from_groups_of_four_where_planned() {
+    const auto write = PerThreadWrite<ND::_2D, float3>::build(image<float3>(0x7000000000ull, 2880, 2160, 34560));
+    const auto chain = [&](size_t address, uint pitch, const Rect& crop, const Size& to) {
+        return PerThreadRead<ND::_2D, uchar3>::build(image<uchar3>(address, 3840, 2160, pitch)).then(Crop<>::build(crop)).then(
+            Resize<InterpolationType::INTER_LINEAR>::build(to));
+    };
+    const auto flags_of = [&](const auto& read) { return exec::JobOf<std::decay_t<decltype(read)>, std::decay_t<decltype(write)>>::make(read, write); };
+    // 1024x576 -> 2048x1152 (1152 tiles of 64 x 32): 34 x 18 source pixels per tile, ten groups per row, 180 groups
+    const auto wide = flags_of(chain(0x1000000000ull, 11520, Rect(8, 8, 1024, 576), Size(2048, 1152)));
+    CHECK(wide.wave_rows == 8u && (wide.flags & exec::FLAG_QUAD_FILL) != 0u && (wide.flags & exec::FLAG_SOURCE_TILE) != 0u);
+    // 2048x1536 -> 2880x2160 (the factors of the headline's planes): 47 x 25 source pixels per tile, 325 groups: one pixel per thread
+    const auto headline = flags_of(chain(0x1000000000ull, 11520, Rect(8, 8, 2048, 1536), Size(2880, 2160)));
+    CHECK(headline.wave_rows == 8u && (headline.flags & exec::FLAG_QUAD_FILL) == 0u && (headline.flags & exec::FLAG_SOURCE_TILE) != 0u);
+    // a small output: 64 x 16 tiles, one pixel per thread
+    const auto small = flags_of(chain(0x1000000000ull, 11520, Rect(8, 8, 100, 60), Size(224, 224)));
+    CHECK(small.wave_rows == 4u && (small.flags & exec::FLAG_QUAD_FILL) == 0u && (small.flags & exec::FLAG_SOURCE_TILE) != 0u);
+    // rows that are not a whole number of dwords apart, an image that does not start at a whole dword
+    CHECK((flags_of(chain(0x1000000000ull, 11521, Rect(8, 8, 1024, 576), Size(2048, 1152))).flags & exec::FLAG_QUAD_FILL) == 0u);
+    CHECK((flags_of(chain(0x1000000002ull, 11520, Rect(8, 8, 1024, 576), Size(2048, 1152))).flags & exec::FLAG_QUAD_FILL) == 0u);
+}
+
 // a batch of windows of different sizes: every plane gets the extent of the batch's thread grid, and the wide (several
 // pixels per thread) path only where the rows below the first are aligned too
 void ragged_batches_take_their_alignment_from_the_whole_box() {
@@ -115,6 +138,7 @@ void tile_pairs_are_a_permutation_with_neighbours_eight_apart() {
 int main() {
     huge_windows_keep_64_bit_addressing();
     tile_pairs_are_a_permutation_with_neighbours_eight_apart();
+    tiles_are_filled_from_groups_of_four_where_planned();
     ragged_batches_take_their_alignment_from_the_whole_box();
     if (failures == 0) std::printf("host plans: ok\n");
     return failures == 0 ? 0 : 1;

@@ -158,12 +158,14 @@ def test_float_tiles_filled_from_groups_of_four_pixels(fk, oracle, width):
     """Up-scaled crops of an image whose rows are a whole number of dwords apart: the tiles of float taps are filled from
     aligned groups of four pixels of the parent image.  Windows that start at every phase of such a group, that end inside
     the parent (the pixel behind the window's last column exists in memory but must not be used: the tap clamps to the
-    window) and at its last column and row (the last group of the last row ends at the end of the allocation)."""
+    window) and at its last column and row (the last group of the last row ends at the end of the allocation).  The
+    640x416 outputs make a launch of more than 1024 tiles of 64x32, which is where the kernel fills its tiles this way; the
+    small ones take the fill of one pixel per thread on the same windows."""
     h = 61
     src = oracle.bytes(83 + width, (h, width, 3))
     rects = [(x, 2 + x, 31 + x, 23) for x in (0, 1, 2, 3, 5)]
     rects += [(width - 29, h - 19, 29, 19), (width - 1, h - 1, 1, 1), (width - 5, 0, 5, h), (0, h - 2, width, 2), (0, 0, width, h)]
-    for dst in ((200, 150), (97, 131)):
+    for dst in ((640, 416), (97, 131)):
         for aspect in (B.IGNORE_AR, B.PRESERVE_AR):
             args = (aspect, (0.5, 0.25, 0.125), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)
             out = torch.full((len(rects), dst[1], dst[0], 3), float("nan"), device="cuda")
