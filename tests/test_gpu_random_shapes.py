@@ -39,6 +39,29 @@ def test_readme_chain(fk, oracle, seed):
         assert same_bits(out.cpu().numpy(), oracle.crop_resize_muls_bgr_tensor(src, rects, dst, *args)), (seed, case, w, h, rects, dst, args[0])
 
 
+@pytest.mark.parametrize("seed", [11, 12])
+def test_readme_chain_large_outputs(fk, oracle, seed):
+    """Launches of more than 1024 tiles, where the kernel takes 64x32 tiles and, for images whose rows are a whole number of
+    dwords apart, fills them from aligned groups of four pixels: image widths that are and are not multiples of four, windows
+    at any offset, up- and down-scaling, all aspect modes."""
+    rng = np.random.default_rng(seed)
+    for case in range(24):
+        w, h = int(rng.integers(40, 900)), int(rng.integers(40, 600))
+        if case % 3 != 2:
+            w = (w + 3) & ~3
+        src = oracle.bytes(int(rng.integers(1, 1 << 30)), (h, w, 3))
+        n = int(rng.integers(2, 6))
+        rects = windows(rng, n, w, h)
+        if case % 2 == 0:  # windows of at least a third of the image: several tiles per source box row
+            rects = [(x, y, max(cw, w // 3), max(ch, h // 3)) for x, y, cw, ch in rects]
+            rects = [(min(x, w - cw), min(y, h - ch), cw, ch) for x, y, cw, ch in rects]
+        dst = (int(rng.integers(640, 1400)), int(rng.integers(520, 900)))
+        args = (int(rng.integers(0, 4)), (1.0, 2.0, 3.0), (1.4,) * 3, (0.5,) * 3, (255.,) * 3)
+        out = torch.empty((n, dst[1], dst[0], 3), device="cuda")
+        fk.crop_resize_muls_bgr_tensor(dev(src), rects, out, *args)
+        assert same_bits(out.cpu().numpy(), oracle.crop_resize_muls_bgr_tensor(src, rects, dst, *args)), (seed, case, w, h, rects, dst, args[0])
+
+
 @pytest.mark.parametrize("seed", [4, 5])
 def test_planar_batch(fk, oracle, seed):
     rng = np.random.default_rng(seed)
