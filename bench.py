@@ -53,12 +53,19 @@ class StreamTimer:
     def start(self):
         assert self.rt.fkrt_event_record(self.a, self.stream) == 0
 
-    def stop_ms(self):
+    def stop(self):
         assert self.rt.fkrt_event_record(self.b, self.stream) == 0
+
+    def elapsed_ms(self):
+        """After the device has been synchronised."""
         assert self.rt.fkrt_event_sync(self.b) == 0
         ms = C.c_float()
         assert self.rt.fkrt_event_elapsed_ms(C.byref(ms), self.a, self.b) == 0
         return float(ms.value)
+
+    def stop_ms(self):
+        self.stop()
+        return self.elapsed_ms()
 
 
 SPINUP_S = 0.2
@@ -113,14 +120,13 @@ def time_blocks(timer, launch, steps, warmup, blocks):
             timer.start()
             for i in range(1, steps):
                 launch(n + i)
-            ev = timer.stop_ms() / (steps - 1)
         else:
             timer.start()
             launch(n)
-            ev = timer.stop_ms()
+        timer.stop()
         torch.cuda.synchronize()
         wall.append((time.perf_counter() - t0) * 1e3 / steps)
-        events.append(ev)
+        events.append(timer.elapsed_ms() / max(1, steps - 1))  # (read after the wall clock has stopped)
         n += steps
     return wall, events
 
